@@ -12,10 +12,10 @@ import os
 from dataclasses import dataclass
 from typing import Callable, Dict
 
-from .specs import (AttentionSpec, ConfigError, EmbeddingSpec, GatedMLPSpec,
-                    HeadSpec, HyperConnectionSpec, LatentAttentionSpec, LayerRun, LayerSpec, MLSTMSpec,
+from .specs import (AttentionSpec, ConfigError, DecayAttentionSpec, EmbeddingSpec, GatedDeltaSpec, GatedMLPSpec,
+                    HeadSpec, HyperConnectionSpec, LatentAttentionSpec, LayerNormSpec, LayerRun, LayerSpec, MLSTMSpec,
                     MixedHeadAttentionSpec, ModelSpec, NoPositionSpec, OnePlusRMSNormSpec, RMSNormSpec, RopeSpec,
-                    ScaledRopeSpec)
+                    RoutedMLPSpec, ScaledRopeSpec)
 
 
 @dataclass(frozen=True)
@@ -104,3 +104,8 @@ from . import rerizen as _rerizen  # noqa: E402
 
 register_architecture(_rerizen.ARCHITECTURE, _rerizen.RerizenConfig.from_dict)
 RerizenConfig = _rerizen.RerizenConfig
+
+from . import bebulorn as _bebulorn  # noqa: E402
+
+register_architecture(_bebulorn.ARCHITECTURE, _bebulorn.BebulornConfig.from_dict)
+BebulornConfig = _bebulorn.BebulornConfig

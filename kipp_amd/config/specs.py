@@ -42,6 +42,18 @@ class OnePlusRMSNormSpec:
 
 
 @dataclass(frozen=True)
+class LayerNormSpec:
+    """y = (x - mean x) / sqrt(var x + eps) * w + b over the last axis of `width`, var the mean of the squared
+    deviations.  `name` and `bias_name`: the tensors' local names (file name = prefix + name)."""
+    width: int
+    eps: float
+    prefix: str = ""
+    name: str = "weight"
+    bias_name: str = "bias"
+    kind: str = "layer_norm"
+
+
+@dataclass(frozen=True)
 class RopeSpec:
     """Rotary position encoding over the first `rotary_dim` dims of a head.
 
@@ -116,6 +128,9 @@ class AttentionSpec:
     `v_head_dim` D: values have D numbers a head (None: as keys).  `own_kv` False: the mixer
     has no key and value projections and reads the cache of another run (`LayerRun.cache_of`).
     `names`: local tensor names of (q, k, v, o, q norm, k norm).
+    `softcap` c: a score s (scale and head factor applied) becomes c tanh(s / c) before the softmax.
+    `head_temp` name: a tensor [heads] of that local name multiplies the scores of each query head.
+    `v_norm_eps`: every head of a value is divided by its root mean square (no weight) before it is cached.
     """
     hidden_size: int
     num_heads: int
@@ -135,10 +150,17 @@ class AttentionSpec:
     own_kv: bool = True
     names: Tuple[str, ...] = ("q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight", "q_norm.weight", "k_norm.weight")
     bias_names: Tuple[str, str, str] = ("q_proj.bias", "k_proj.bias", "v_proj.bias")
+    softcap: Optional[float] = None
+    head_temp: Optional[str] = None
+    v_norm_eps: Optional[float] = None
 
     def __post_init__(self):
         if self.num_heads <= 0 or self.num_kv_heads <= 0:
             raise ConfigError("attention needs at least one query head and one key/value head")
+        if self.softcap is not None and not self.softcap > 0:
+            raise ConfigError(f"attention softcap must be positive, got {self.softcap}")
+        if self.v_norm_eps is not None and not self.v_norm_eps >= 0:
+            raise ConfigError(f"attention v_norm_eps must not be negative, got {self.v_norm_eps}")
         if self.v_head_dim is not None and not 0 < self.v_head_dim <= 256:
             raise ConfigError(f"value head size {self.v_head_dim} unsupported: from 1 to 256")
         if self.q_temp is not None and not (len(self.q_temp) == 2 and isinstance(self.q_temp[1], int) and self.q_temp[1] > 0):
@@ -182,7 +204,8 @@ class AttentionSpec:
     @property
     def plain(self) -> bool:
         """None of the extras: the mixer's first kernels (weighted norm, rotation, fused decode) apply."""
-        return not self.bias and self.qk_norm_weight and self.q_temp is None and self.v_head_dim is None and self.own_kv
+        return not self.bias and self.qk_norm_weight and self.q_temp is None and self.v_head_dim is None and self.own_kv \
+            and self.softcap is None and self.head_temp is None and self.v_norm_eps is None
 
 
 @dataclass(frozen=True)
@@ -259,6 +282,73 @@ class MLSTMSpec:
             raise ConfigError(f"mlstm: gate_cap must be positive, got {self.gate_cap}")
         if len(self.names) != 10:
             raise ConfigError("names: ten local tensor names")
+
+
+@dataclass(frozen=True)
+class DecayAttentionSpec:
+    """Linear attention with a fixed decay a head (lightning attention): per head a state S [head_dim, v_head_dim] that
+    starts at zero and is carried from token to token in float32.
+
+    q = silu(W_q x), k = silu(W_k x), v = silu(W_v x);  S_t = decay_h S_(t-1) + k_t v_t^T;  o_t = S_t^T q_t;
+    all heads of o side by side over their root mean square (`norm_eps`), times the norm weight [heads v_head_dim],
+    times sigmoid(W_g x), then W_o.  `decays`: one number a head.  `names`: local tensor names of (q, k, v, g, o, norm)."""
+    hidden_size: int
+    num_heads: int
+    head_dim: int
+    v_head_dim: int
+    decays: Tuple[float, ...]
+    norm_eps: float
+    prefix: str = ""
+    kind: str = "decay_attention"
+    names: Tuple[str, ...] = ("q", "k", "v", "g", "o", "norm")
+
+    def __post_init__(self):
+        if self.num_heads <= 0 or self.v_head_dim <= 0 or not 0 < self.head_dim <= 1024:
+            raise ConfigError("decay attention: heads and value size must be positive, key size from 1 to 1,024")
+        if len(self.decays) != self.num_heads:
+            raise ConfigError(f"decay attention: {len(self.decays)} decays for {self.num_heads} heads")
+        if len(self.names) != 6:
+            raise ConfigError("names: six local tensor names")
+
+
+@dataclass(frozen=True)
+class GatedDeltaSpec:
+    """The gated delta rule: per head a state S [head_dim, v_head_dim] that starts at zero and is carried from token to
+    token in float32, beside the last `conv_taps` - 1 inputs of the short convolutions.
+
+    q = W_q x and k = W_k x (`num_kv_heads` heads of head_dim), v = W_v x (`num_heads` heads of v_head_dim); head h reads
+    q/k head h // (num_heads / num_kv_heads).  Each channel of q, k and v passes a causal filter over its last
+    `conv_taps` inputs (zeros before the start, the last tap is the current token's) and silu; every head of q and k is
+    divided by sqrt(sum x^2 + `unit_eps`), q also by sqrt(head_dim).  beta = sigmoid(W_b x) and
+    g = exp(-exp(A_h) softplus(W_a x + dt_h)), one a head.  S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.
+    Every head of o over its root mean square (`norm_eps`), times the norm weight [v_head_dim], times silu(W_g x), then W_o.
+    `names`: local tensor names of (q, k, v, q filter, k filter, v filter, b, a, A, dt, g, o, norm)."""
+    hidden_size: int
+    num_heads: int
+    num_kv_heads: int
+    head_dim: int
+    v_head_dim: int
+    conv_taps: int
+    norm_eps: float
+    unit_eps: float = 1e-6
+    prefix: str = ""
+    kind: str = "gated_delta"
+    names: Tuple[str, ...] = ("q", "k", "v", "q.conv", "k.conv", "v.conv", "b", "a", "A_log", "dt_bias", "g", "o", "norm")
+
+    def __post_init__(self):
+        if self.num_heads <= 0 or self.num_kv_heads <= 0 or self.num_heads % self.num_kv_heads:
+            raise ConfigError(f"gated delta: heads {self.num_heads} must be a positive multiple of q/k heads {self.num_kv_heads}")
+        if self.v_head_dim <= 0 or not 0 < self.head_dim <= 1024:
+            raise ConfigError("gated delta: value size must be positive, key size from 1 to 1,024")
+        if not 1 <= self.conv_taps <= 16:
+            raise ConfigError(f"gated delta: the short convolution takes 1 to 16 taps, got {self.conv_taps}")
+        if len(self.names) != 13:
+            raise ConfigError("names: thirteen local tensor names")
+
+    @property
+    def channels(self) -> int:
+        """Channels that pass a short convolution: q | k | v."""
+        return 2 * self.num_kv_heads * self.head_dim + self.num_heads * self.v_head_dim
 
 
 @dataclass(frozen=True)
@@ -343,7 +433,7 @@ class MixedHeadAttentionSpec:
 
 @dataclass(frozen=True)
 class GatedMLPSpec:
-    """down(act(gate(x)) * up(x)); `activation` is "silu".  `names`: the local tensor names of (gate, up, down)."""
+    """down(act(gate(x)) * up(x)); `activation` is "silu" or "relu".  `names`: the local tensor names of (gate, up, down)."""
     hidden_size: int
     intermediate_size: int
     activation: str = "silu"
@@ -354,8 +444,40 @@ class GatedMLPSpec:
     def __post_init__(self):
         if self.intermediate_size <= 0:
             raise ConfigError("intermediate_size must be positive")
-        if self.activation != "silu":
-            raise ConfigError(f"activation {self.activation!r} unsupported (silu only)")
+        if self.activation not in ("silu", "relu"):
+            raise ConfigError(f"activation {self.activation!r} unsupported (silu, relu)")
+
+
+@dataclass(frozen=True)
+class RoutedMLPSpec:
+    """A mixture of `experts` small feed-forwards, of which a token uses `top`: W_down_e act(W_up_e x), `activation`
+    "gelu" (the exact one, with erf), "gelu_tanh", "silu" or "relu".  p = softmax(W_router x) over all experts in float32; the
+    `top` largest are chosen (the lower index first among equals) and weigh their experts' results by p / (sum of the
+    chosen p + `weight_eps`).  `shared_size` I: one more expert of inner size I (tensors under `shared_prefix`) runs for
+    every token and is added (None: none).  Expert e's tensors are `expert_prefix.format(e)` + (up, down)."""
+    hidden_size: int
+    experts: int
+    top: int
+    expert_size: int
+    shared_size: Optional[int] = None
+    activation: str = "gelu"
+    weight_eps: float = 1e-20
+    prefix: str = ""
+    kind: str = "routed_mlp"
+    router_name: str = "router"
+    expert_prefix: str = "e{}."
+    shared_prefix: str = "shared."
+    names: Tuple[str, str] = ("up", "down")
+
+    def __post_init__(self):
+        if not 0 < self.top <= self.experts:
+            raise ConfigError(f"routed feed-forward: top {self.top} must be from 1 to experts {self.experts}")
+        if self.experts > 1024 or self.top > 32:
+            raise ConfigError("routed feed-forward: up to 1,024 experts, up to 32 a token")
+        if self.expert_size <= 0 or (self.shared_size is not None and self.shared_size <= 0):
+            raise ConfigError("routed feed-forward: inner sizes must be positive")
+        if self.activation not in ("gelu", "gelu_tanh", "silu", "relu"):
+            raise ConfigError(f"activation {self.activation!r} unsupported (gelu, gelu_tanh, silu, relu)")
 
 
 @dataclass(frozen=True)
@@ -369,7 +491,9 @@ class LayerSpec:
     a = `residual_scale`; "post_norm_mixer" is its first half alone.  "hyper_pre_norm" keeps
     several copies of the residual stream and has the roles mixer_norm, mixer_hc, mixer,
     ffn_norm, ffn_hc, ffn (the *_hc parts say how a sublayer reads and writes the copies);
-    "hyper_pre_norm_mixer" is its first half alone.
+    "hyper_pre_norm_mixer" is its first half alone.  "sandwich_norm" norms a sublayer's input and its result:
+    x += a mixer_post_norm(mixer(mixer_norm(x))); x += a ffn_post_norm(ffn(ffn_norm(x))), a = `residual_scale`;
+    "sandwich_norm_mixer" is its first half alone.
     """
     parts: Tuple[Tuple[str, object], ...]
     block: str = "pre_norm"
@@ -390,9 +514,11 @@ class LayerSpec:
 class LayerRun:
     """One entry of the run order: run `layer`; `cache_of` names an earlier
     entry of the order (by index) whose cache this run reads instead of
-    writing its own."""
+    writing its own.  `add_embedding`: the embedding's output (the residual stream as it was before the first run)
+    is added to the residual stream right before this run."""
     layer: int
     cache_of: Optional[int] = None
+    add_embedding: bool = False
 
 
 @dataclass(frozen=True)

@@ -6,7 +6,7 @@
 // float32 path's kernel and the fallback of sizes the MFMA kernels refuse.
 //
 // For query position p of a sequence the keys are s in [max(0, p-window+1), p]
-// (window 0: from 0), score = (q . k_s) * scale, softmax with the maximum
+// (window 0: from 0), score = (q . k_s) * scale (with `softcap` c > 0: c tanh(score / c)), softmax with the maximum
 // subtracted, out = sum p_s v_s  (/root/reference/src/kipp.c:2882-2922).  Keys are
 // taken in tiles of 64 aligned to absolute key index, so the sequence of
 // operations for one query depends on its own position only, never on what
@@ -57,7 +57,7 @@ __global__ void paged_attention_generic_kernel(
     const TQ* __restrict__ q, const TC* __restrict__ k_cache, const TC* __restrict__ v_cache, TO* __restrict__ out,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
     const int32_t* __restrict__ block_table, int max_blocks,
-    int n_q, int n_kv, int d, int dv, int v_row, int page, float scale, int window) {
+    int n_q, int n_kv, int d, int dv, int v_row, int page, float scale, int window, float softcap) {
     __shared__ float q_s[HEADS_PER_BLOCK][MAX_D];
     __shared__ float p_s[HEADS_PER_BLOCK][KIPP_WAVE];
     __shared__ unsigned long long off_s[HEADS_PER_BLOCK][KIPP_WAVE];
@@ -92,6 +92,7 @@ __global__ void paged_attention_generic_kernel(
             off = ((unsigned long long)page_id * n_kv + g) * page + s % page;
             const TC* k_row = k_cache + off * d;
             score = dot_row(q_s[wave], k_row, d) * scale;
+            if (softcap > 0.0f) score = softcap * tanhf(score / softcap);
         }
         const float m_new = fmaxf(m, wave_max(score));
         const float alpha = expf(m - m_new);
@@ -130,22 +131,31 @@ __global__ void paged_attention_generic_kernel(
 }
 
 // Values of width dv in rows of v_row numbers (v_row = dv for a value cache of its own).
-extern "C" int kipp_paged_attention_generic_v(
+extern "C" int kipp_paged_attention_generic_capped(
     const void* q, int q_dtype, const void* k_cache, const void* v_cache, int cache_dtype, void* out, int out_dtype,
     const int32_t* positions, const int32_t* seq_of_token, const int32_t* block_table, int max_blocks,
-    int n_tokens, int n_q, int n_kv, int d, int dv, int v_row, int page, float scale, int window, hipStream_t stream) {
+    int n_tokens, int n_q, int n_kv, int d, int dv, int v_row, int page, float scale, int window, float softcap,
+    hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (d > MAX_D || d <= 0 || dv > MAX_D || dv <= 0 || v_row < dv || n_kv <= 0 || n_q % n_kv) return -1;
     dim3 grid((n_q + HEADS_PER_BLOCK - 1) / HEADS_PER_BLOCK, n_tokens), block(HEADS_PER_BLOCK * KIPP_WAVE);
 #define KIPP_PA(TQ, TC, TO)                                                                                    \
     hipLaunchKernelGGL((paged_attention_generic_kernel<TQ, TC, TO>), grid, block, 0, stream, (const TQ*)q,     \
                        (const TC*)k_cache, (const TC*)v_cache, (TO*)out, positions, seq_of_token, block_table, \
-                       max_blocks, n_q, n_kv, d, dv, v_row, page, scale, window)
+                       max_blocks, n_q, n_kv, d, dv, v_row, page, scale, window, softcap)
     if (q_dtype == KIPP_F32 && cache_dtype == KIPP_F32 && out_dtype == KIPP_F32) KIPP_PA(float, float, float);
     else if (q_dtype == KIPP_BF16 && cache_dtype == KIPP_BF16 && out_dtype == KIPP_BF16) KIPP_PA(bf16_t, bf16_t, bf16_t);
     else return -2;
 #undef KIPP_PA
     return KIPP_LAUNCH_CHECK();
+}
+
+extern "C" int kipp_paged_attention_generic_v(
+    const void* q, int q_dtype, const void* k_cache, const void* v_cache, int cache_dtype, void* out, int out_dtype,
+    const int32_t* positions, const int32_t* seq_of_token, const int32_t* block_table, int max_blocks,
+    int n_tokens, int n_q, int n_kv, int d, int dv, int v_row, int page, float scale, int window, hipStream_t stream) {
+    return kipp_paged_attention_generic_capped(q, q_dtype, k_cache, v_cache, cache_dtype, out, out_dtype, positions, seq_of_token,
+                                               block_table, max_blocks, n_tokens, n_q, n_kv, d, dv, v_row, page, scale, window, 0.0f, stream);
 }
 
 extern "C" int kipp_paged_attention_generic(

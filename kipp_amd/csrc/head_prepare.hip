@@ -8,6 +8,8 @@
 //     bias    u += bias[column]                               (bias over the q | k | v columns, or none)
 //     norm    u *= rsqrt(mean(u^2) + eps) [* w]               (queries and keys; mode 0 none, 1 plain, 2 weighted)
 //     factor  queries at position p times 1 + coef * ln(floor((p + 1) / every) + 1)     (every 0: none)
+//     head    queries of head h times q_head_scale[h]                                    (or none)
+//     values  every value head over its root mean square, rsqrt(mean(u^2) + v_norm_eps)  (v_norm_eps < 0: none)
 //     write   q to q_out [tokens][n_q d]; the key and value of position p to page table[p / page], slot p % page;
 //             caches [page][kv head][slot][d] and [page][kv head][slot][dv]
 // All arithmetic is float32.
@@ -24,7 +26,7 @@ __global__ void head_prepare_kernel(
     const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
     const int32_t* __restrict__ block_table, int max_blocks, int norm_mode, const float* __restrict__ q_norm_w,
     const float* __restrict__ k_norm_w, float eps, float temp_coef, int temp_every,
-    int n_q, int n_kv, int d, int dv, int page, int write_kv) {
+    int n_q, int n_kv, int d, int dv, int page, int write_kv, const float* __restrict__ q_head_scale, float v_norm_eps) {
     const int wave = threadIdx.x / KIPP_WAVE;
     const int lane = threadIdx.x & (KIPP_WAVE - 1);
     const int t = blockIdx.y;
@@ -67,6 +69,16 @@ __global__ void head_prepare_kernel(
 #pragma unroll
         for (int c = 0; c < MAX_D / KIPP_WAVE; ++c) vals[c] *= factor;
     }
+    if (kind == 0 && q_head_scale != nullptr) {
+        const float factor = q_head_scale[head];
+#pragma unroll
+        for (int c = 0; c < MAX_D / KIPP_WAVE; ++c) vals[c] *= factor;
+    }
+    if (kind == 2 && v_norm_eps >= 0.0f) {
+        const float scale = 1.0f / sqrtf(wave_sum(ss) / (float)dv + v_norm_eps);
+#pragma unroll
+        for (int c = 0; c < MAX_D / KIPP_WAVE; ++c) vals[c] *= scale;
+    }
     if (kind == 0) {
         TO* dst = q_out + ((size_t)t * n_q + head) * d;
 #pragma unroll
@@ -86,11 +98,12 @@ __global__ void head_prepare_kernel(
     }
 }
 
-extern "C" int kipp_head_prepare(
+extern "C" int kipp_head_prepare_scaled(
     const float* proj, int parts, int stride, const float* bias, void* q_out, int q_dtype, void* k_cache, void* v_cache,
     int cache_dtype, const int32_t* positions, const int32_t* seq_of_token, const int32_t* block_table, int max_blocks,
     int norm_mode, const float* q_norm_w, const float* k_norm_w, float eps, float temp_coef, int temp_every,
-    int n_tokens, int n_q, int n_kv, int d, int dv, int page, int write_kv, hipStream_t stream) {
+    int n_tokens, int n_q, int n_kv, int d, int dv, int page, int write_kv, const float* q_head_scale, float v_norm_eps,
+    hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (d <= 0 || d > MAX_D || dv <= 0 || dv > MAX_D || n_q <= 0 || n_kv <= 0 || page <= 0) return -1;
     if (stride < n_q * d + (write_kv ? n_kv * (d + dv) : 0) || norm_mode < 0 || norm_mode > 2 || temp_every < 0) return -1;
@@ -101,10 +114,21 @@ extern "C" int kipp_head_prepare(
 #define KIPP_HP(TO, TC)                                                                                              \
     hipLaunchKernelGGL((head_prepare_kernel<TO, TC>), grid, block, 0, stream, proj, parts, part_stride, stride, bias, \
                        (TO*)q_out, (TC*)k_cache, (TC*)v_cache, positions, seq_of_token, block_table, max_blocks,      \
-                       norm_mode, q_norm_w, k_norm_w, eps, temp_coef, temp_every, n_q, n_kv, d, dv, page, write_kv)
+                       norm_mode, q_norm_w, k_norm_w, eps, temp_coef, temp_every, n_q, n_kv, d, dv, page, write_kv,     \
+                       q_head_scale, v_norm_eps)
     if (q_dtype == KIPP_F32 && cache_dtype == KIPP_F32) KIPP_HP(float, float);
     else if (q_dtype == KIPP_BF16 && cache_dtype == KIPP_BF16) KIPP_HP(bf16_t, bf16_t);
     else return -2;
 #undef KIPP_HP
     return KIPP_LAUNCH_CHECK();
+}
+
+extern "C" int kipp_head_prepare(
+    const float* proj, int parts, int stride, const float* bias, void* q_out, int q_dtype, void* k_cache, void* v_cache,
+    int cache_dtype, const int32_t* positions, const int32_t* seq_of_token, const int32_t* block_table, int max_blocks,
+    int norm_mode, const float* q_norm_w, const float* k_norm_w, float eps, float temp_coef, int temp_every,
+    int n_tokens, int n_q, int n_kv, int d, int dv, int page, int write_kv, hipStream_t stream) {
+    return kipp_head_prepare_scaled(proj, parts, stride, bias, q_out, q_dtype, k_cache, v_cache, cache_dtype, positions, seq_of_token,
+                                    block_table, max_blocks, norm_mode, q_norm_w, k_norm_w, eps, temp_coef, temp_every, n_tokens, n_q,
+                                    n_kv, d, dv, page, write_kv, nullptr, -1.0f, stream);
 }

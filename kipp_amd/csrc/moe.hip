@@ -1,0 +1,261 @@
+// A routed feed-forward (mixture of experts): the router's choice, the tokens sorted by expert, the experts'
+// two products over those runs of rows, and the weighted sum.
+//
+//     route    p = softmax(z) over all experts (float32); the `top` largest p (the lower index first among equals);
+//              weight = p / (sum of the chosen p + eps)
+//     sort     the (token, choice) pairs in runs of one expert each, cut into tiles of up to 16 rows; the list of tiles
+//              is made on the device, so the host never learns the counts and the launches have a fixed shape
+//     expert   a tile's rows against its expert's matrix: out[row][n] = act(sum_k W_e[n][k] x[row][k]); a lane takes a
+//              column, the sum over k runs in index order, so a row's result does not depend on its tile
+//     combine  out[t] = sum_j weight[t][j] y[place of (t, j)] (+ the shared expert's result, slabs added in order)
+#include "common.h"
+#include <math.h>
+
+#define ROUTE_WAVES 4
+#define MAX_EXPERTS 1024
+#define MAX_TOP 32
+#define TILE_ROWS 16
+#define EXPERT_COLS 256
+#define EXPERT_KC 128
+
+enum { ACT_NONE = -1, ACT_SILU = 0, ACT_RELU = 1, ACT_GELU = 2, ACT_GELU_TANH = 3 };
+
+__device__ __forceinline__ float activate(float z, int act) {
+    switch (act) {
+        case ACT_SILU: return z / (1.0f + expf(-z));
+        case ACT_RELU: return fmaxf(z, 0.0f);
+        case ACT_GELU: return 0.5f * z * (1.0f + erff(z * 0.70710678118654752440f));
+        case ACT_GELU_TANH: return 0.5f * z * (1.0f + tanhf(0.79788456080286535588f * (z + 0.044715f * z * z * z)));
+        default: return z;
+    }
+}
+
+// One wave a token.  z: float32 [tokens][stride] (or slabs of it, added in order).
+__global__ void __launch_bounds__(ROUTE_WAVES * KIPP_WAVE)
+moe_route_kernel(const float* __restrict__ z, int parts, size_t part_stride, int stride, int32_t* __restrict__ chosen,
+                 float* __restrict__ weight, int tokens, int experts, int top, float eps) {
+    const int wave = threadIdx.x / KIPP_WAVE, lane = threadIdx.x & (KIPP_WAVE - 1);
+    const int t = blockIdx.x * ROUTE_WAVES + wave;
+    if (t >= tokens) return;        // no barrier below
+    float p[MAX_EXPERTS / KIPP_WAVE];
+    float m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < MAX_EXPERTS / KIPP_WAVE; ++i) {
+        const int e = lane + i * KIPP_WAVE;
+        float v = -INFINITY;
+        if (e < experts) {
+            v = z[(size_t)t * stride + e];
+            for (int q = 1; q < parts; ++q) v += z[q * part_stride + (size_t)t * stride + e];
+        }
+        p[i] = v;
+        m = fmaxf(m, v);
+    }
+    m = wave_max(m);
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < MAX_EXPERTS / KIPP_WAVE; ++i) {
+        p[i] = (lane + i * KIPP_WAVE < experts) ? expf(p[i] - m) : -1.0f;
+        if (p[i] > 0.0f) sum += p[i];
+    }
+    sum = wave_sum(sum);
+    float picked_sum = 0.0f;
+    float mine = 0.0f;          // lane j keeps the j-th choice
+    int mine_e = 0;
+    for (int j = 0; j < top; ++j) {
+        float best = -1.0f;
+        int best_e = MAX_EXPERTS;
+#pragma unroll
+        for (int i = 0; i < MAX_EXPERTS / KIPP_WAVE; ++i)
+            if (p[i] > best) { best = p[i]; best_e = lane + i * KIPP_WAVE; }     // the lowest index of a lane's largest
+        for (int off = 32; off > 0; off >>= 1) {
+            const float ob = __shfl_xor(best, off, KIPP_WAVE);
+            const int oe = __shfl_xor(best_e, off, KIPP_WAVE);
+            if (ob > best || (ob == best && oe < best_e)) { best = ob; best_e = oe; }
+        }
+#pragma unroll
+        for (int i = 0; i < MAX_EXPERTS / KIPP_WAVE; ++i)
+            if (lane + i * KIPP_WAVE == best_e) p[i] = -1.0f;
+        const float s = best / sum;
+        picked_sum += s;
+        if (lane == j) { mine = s; mine_e = best_e; }
+    }
+    if (lane < top) {
+        chosen[(size_t)t * top + lane] = mine_e;
+        weight[(size_t)t * top + lane] = mine / (picked_sum + eps);
+    }
+}
+
+// One workgroup sorts all pairs.  tiles: int32 [max_tiles][3] = (expert, first row, rows); rows 0 marks an unused tile.
+__global__ void __launch_bounds__(1024)
+moe_sort_kernel(const int32_t* __restrict__ chosen, int pairs, int experts, int top, int32_t* __restrict__ pair_token,
+                int32_t* __restrict__ place_of_pair, int32_t* __restrict__ tiles, int max_tiles) {
+    __shared__ int count[MAX_EXPERTS];
+    __shared__ int first[MAX_EXPERTS + 1];
+    __shared__ int tile_first[MAX_EXPERTS + 1];
+    for (int e = threadIdx.x; e < experts; e += blockDim.x) count[e] = 0;
+    __syncthreads();
+    for (int p = threadIdx.x; p < pairs; p += blockDim.x) atomicAdd(&count[chosen[p]], 1);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int rows = 0, tl = 0;
+        for (int e = 0; e < experts; ++e) {
+            first[e] = rows;
+            tile_first[e] = tl;
+            rows += count[e];
+            tl += (count[e] + TILE_ROWS - 1) / TILE_ROWS;
+        }
+        first[experts] = rows;
+        tile_first[experts] = tl;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < experts; e += blockDim.x) {
+        const int n = count[e];
+        for (int j = 0; j * TILE_ROWS < n; ++j) {
+            int32_t* tile = tiles + (size_t)(tile_first[e] + j) * 3;
+            tile[0] = e;
+            tile[1] = first[e] + j * TILE_ROWS;
+            tile[2] = min(TILE_ROWS, n - j * TILE_ROWS);
+        }
+    }
+    for (int i = tile_first[experts] + threadIdx.x; i < max_tiles; i += blockDim.x) {
+        tiles[(size_t)i * 3] = 0;
+        tiles[(size_t)i * 3 + 1] = 0;
+        tiles[(size_t)i * 3 + 2] = 0;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < experts; e += blockDim.x) count[e] = 0;     // now the next free place of a run
+    __syncthreads();
+    for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+        const int e = chosen[p];
+        const int at = first[e] + atomicAdd(&count[e], 1);
+        pair_token[at] = p / top;
+        place_of_pair[p] = at;
+    }
+}
+
+// x rows are x[gather[row]] (gather null: x[row]); w: [experts][n_out][k]; out[row][n_out].
+template <typename TX, typename TW, typename TO>
+__global__ void __launch_bounds__(EXPERT_COLS)
+moe_expert_kernel(const TX* __restrict__ x, const int32_t* __restrict__ gather, const TW* __restrict__ w,
+                  const int32_t* __restrict__ tiles, TO* __restrict__ out, int n_out, int k, int act) {
+    __shared__ float x_s[TILE_ROWS][EXPERT_KC];
+    const int32_t* tile = tiles + (size_t)blockIdx.x * 3;
+    const int rows = tile[2];
+    if (rows == 0) return;      // uniform over the workgroup
+    const int expert = tile[0], row0 = tile[1];
+    const int col = blockIdx.y * EXPERT_COLS + threadIdx.x;
+    const TW* w_row = w + ((size_t)expert * n_out + (col < n_out ? col : 0)) * k;
+    float acc[TILE_ROWS];
+#pragma unroll
+    for (int r = 0; r < TILE_ROWS; ++r) acc[r] = 0.0f;
+    for (int k0 = 0; k0 < k; k0 += EXPERT_KC) {
+        const int kc = min(EXPERT_KC, k - k0);
+        __syncthreads();
+        for (int i = threadIdx.x; i < TILE_ROWS * EXPERT_KC; i += EXPERT_COLS) {
+            const int r = i / EXPERT_KC, e = i - r * EXPERT_KC;
+            float v = 0.0f;
+            if (r < rows && e < kc) {
+                const size_t src_row = gather != nullptr ? (size_t)gather[row0 + r] : (size_t)(row0 + r);
+                v = load_f(x + src_row * k, k0 + e);
+            }
+            x_s[r][e] = v;
+        }
+        __syncthreads();
+        if (col < n_out) {
+            for (int e = 0; e < kc; ++e) {
+                const float wv = load_f(w_row, k0 + e);
+#pragma unroll
+                for (int r = 0; r < TILE_ROWS; ++r) acc[r] = fmaf(wv, x_s[r][e], acc[r]);
+            }
+        }
+    }
+    if (col >= n_out) return;
+#pragma unroll
+    for (int r = 0; r < TILE_ROWS; ++r)
+        if (r < rows) store_f(out + (size_t)(row0 + r) * n_out, col, activate(acc[r], act));
+}
+
+// out[t][c] = sum_j weight[t][j] y[place[t top + j]][c] + sum of the slabs of shared[t][c]
+__global__ void moe_combine_kernel(const float* __restrict__ y, const int32_t* __restrict__ place, const float* __restrict__ weight,
+                                   const float* __restrict__ shared, int shared_parts, size_t shared_stride,
+                                   float* __restrict__ out, int tokens, int width, int top) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)tokens * width) return;
+    const int t = (int)(i / width), c = (int)(i - (size_t)t * width);
+    float acc = 0.0f;
+    for (int j = 0; j < top; ++j)
+        acc = fmaf(weight[(size_t)t * top + j], y[(size_t)place[(size_t)t * top + j] * width + c], acc);
+    for (int p = 0; p < shared_parts; ++p) acc += shared[p * shared_stride + i];
+    out[i] = acc;
+}
+
+extern "C" int kipp_moe_route(const float* z, int parts, int stride, int32_t* chosen, float* weight, int tokens, int experts, int top,
+                              float eps, int32_t* pair_token, int32_t* place_of_pair, int32_t* tiles, int max_tiles, hipStream_t stream) {
+    if (tokens <= 0) return 0;
+    if (experts <= 0 || experts > MAX_EXPERTS || top <= 0 || top > MAX_TOP || top > experts || stride < experts || parts <= 0) return -1;
+    const int pairs = tokens * top;
+    if (max_tiles < (pairs + TILE_ROWS - 1) / TILE_ROWS + (experts < pairs ? experts : pairs)) return -1;
+    hipLaunchKernelGGL(moe_route_kernel, dim3((tokens + ROUTE_WAVES - 1) / ROUTE_WAVES), dim3(ROUTE_WAVES * KIPP_WAVE), 0, stream, z, parts,
+                       (size_t)tokens * stride, stride, chosen, weight, tokens, experts, top, eps);
+    hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, stream, (const int32_t*)chosen, pairs, experts, top, pair_token,
+                       place_of_pair, tiles, max_tiles);
+    return KIPP_LAUNCH_CHECK();
+}
+
+extern "C" int kipp_moe_expert(const void* x, int x_dtype, const int32_t* gather, const void* w, int w_dtype, const int32_t* tiles,
+                               int max_tiles, void* out, int out_dtype, int n_out, int k, int act, hipStream_t stream) {
+    if (max_tiles <= 0) return 0;
+    if (n_out <= 0 || k <= 0 || act < ACT_NONE || act > ACT_GELU_TANH) return -1;
+    dim3 grid(max_tiles, (n_out + EXPERT_COLS - 1) / EXPERT_COLS), block(EXPERT_COLS);
+#define KIPP_ME(TX, TW, TO)                                                                                                  \
+    hipLaunchKernelGGL((moe_expert_kernel<TX, TW, TO>), grid, block, 0, stream, (const TX*)x, gather, (const TW*)w, tiles, \
+                       (TO*)out, n_out, k, act)
+    if (x_dtype == KIPP_F32 && w_dtype == KIPP_F32 && out_dtype == KIPP_F32) KIPP_ME(float, float, float);
+    else if (x_dtype == KIPP_BF16 && w_dtype == KIPP_BF16 && out_dtype == KIPP_BF16) KIPP_ME(bf16_t, bf16_t, bf16_t);
+    else if (x_dtype == KIPP_BF16 && w_dtype == KIPP_BF16 && out_dtype == KIPP_F32) KIPP_ME(bf16_t, bf16_t, float);
+    else return -2;
+#undef KIPP_ME
+    return KIPP_LAUNCH_CHECK();
+}
+
+extern "C" int kipp_moe_combine(const float* y, const int32_t* place, const float* weight, const float* shared, int shared_parts,
+                                float* out, int tokens, int width, int top, hipStream_t stream) {
+    if (tokens <= 0) return 0;
+    const size_t total = (size_t)tokens * width;
+    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, y, place, weight, shared,
+                       shared != nullptr ? shared_parts : 0, total, out, tokens, width, top);
+    return KIPP_LAUNCH_CHECK();
+}
+
+// out[r][i] = act(sum of the slabs of u[r][i]) [* sum of the slabs of u[r][inner + i] when `glu`]
+template <typename TO>
+__global__ void activate_kernel(const float* __restrict__ u, int parts, size_t part_stride, TO* __restrict__ out, size_t total,
+                                int inner, int glu, int act) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const size_t r = i / inner;
+    const int c = (int)(i - r * inner);
+    const size_t at = glu ? r * 2 * inner + c : i;
+    float a = u[at], b = glu ? u[at + inner] : 1.0f;
+    for (int p = 1; p < parts; ++p) {
+        a += u[p * part_stride + at];
+        if (glu) b += u[p * part_stride + at + inner];
+    }
+    store_f(out, i, glu ? activate(a, act) * b : activate(a, act));
+}
+
+extern "C" int kipp_activate(const float* u, int parts, void* out, int out_dtype, int rows, int inner, int glu, int act,
+                             hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (inner <= 0 || parts <= 0 || act < ACT_SILU || act > ACT_GELU_TANH) return -1;
+    const size_t total = (size_t)rows * inner;
+    const size_t part_stride = total * (glu ? 2 : 1);
+    dim3 grid((unsigned)((total + 255) / 256)), block(256);
+    if (out_dtype == KIPP_F32)
+        hipLaunchKernelGGL((activate_kernel<float>), grid, block, 0, stream, u, parts, part_stride, (float*)out, total, inner, glu, act);
+    else if (out_dtype == KIPP_BF16)
+        hipLaunchKernelGGL((activate_kernel<bf16_t>), grid, block, 0, stream, u, parts, part_stride, (bf16_t*)out, total, inner, glu, act);
+    else
+        return -2;
+    return KIPP_LAUNCH_CHECK();
+}

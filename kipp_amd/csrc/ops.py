@@ -399,12 +399,18 @@ def head_prepare(proj: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor,
                  positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
                  n_q: int, n_kv: int, d: int, dv: int, bias: Optional[torch.Tensor], norm: str, eps: float,
                  q_norm_w: Optional[torch.Tensor] = None, k_norm_w: Optional[torch.Tensor] = None,
-                 temp_coef: float = 0.0, temp_every: int = 0, write_kv: bool = True) -> torch.Tensor:
+                 temp_coef: float = 0.0, temp_every: int = 0, write_kv: bool = True,
+                 q_head_scale: Optional[torch.Tensor] = None, v_norm_eps: Optional[float] = None) -> torch.Tensor:
     """From a step's input product `proj` (float32 [tokens, >= n_q d + n_kv d + n_kv dv], columns q | k | v | ..., or slabs
     of it): `bias` added (float32 over the q | k | v columns), every head of q and k RMS-normed (`norm`: "none", "plain"
     or "weighted" with `q_norm_w` / `k_norm_w` [d]), queries at position p times 1 + temp_coef ln(floor((p + 1) /
-    temp_every) + 1) (temp_every 0: none), q kept in `q_out`, k and v written into the pages of their positions."""
-    _dev(proj, q_out, k_cache, v_cache, positions, seq_of_token, block_table, bias, q_norm_w, k_norm_w)
+    temp_every) + 1) (temp_every 0: none), queries of head h times `q_head_scale[h]` (float32 [n_q]), every value head over
+    its root mean square with `v_norm_eps` inside the root (None: values as they are), q kept in `q_out`, k and v written
+    into the pages of their positions."""
+    _dev(proj, q_out, k_cache, v_cache, positions, seq_of_token, block_table, bias, q_norm_w, k_norm_w, q_head_scale)
+    if q_head_scale is not None:
+        _need(q_head_scale.dtype == torch.float32 and q_head_scale.numel() == n_q, "head_prepare: float32 q_head_scale [n_q]")
+    _need(v_norm_eps is None or v_norm_eps >= 0, "head_prepare: v_norm_eps must not be negative")
     for t, name in ((positions, "positions"), (seq_of_token, "seq_of_token"), (block_table, "block_table")):
         _i32(t, name)
     parts, n, stride = _slabs(proj, "head_prepare")
@@ -421,21 +427,23 @@ def head_prepare(proj: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor,
           and k_cache.shape[3] == d and v_cache.shape[3] == dv and k_cache.dtype == v_cache.dtype,
           "head_prepare: caches must be [pages, n_kv, page, d] and [pages, n_kv, page, dv]")
     _need(block_table.dim() == 2 and int(temp_every) >= 0, "head_prepare: block_table is [sequences, blocks]")
-    fn = _fn("head_prepare", "kipp_head_prepare",
+    fn = _fn("head_prepare", "kipp_head_prepare_scaled",
              [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
-              _c_int, _c_ptr, _c_ptr, _c_float, _c_float, _c_int] + [_c_int] * 7 + [_c_ptr])
+              _c_int, _c_ptr, _c_ptr, _c_float, _c_float, _c_int] + [_c_int] * 7 + [_c_ptr, _c_float, _c_ptr])
     _check(fn(_ptr(proj), parts, stride, _ptr(bias), _ptr(q_out), _code(q_out), _ptr(k_cache), _ptr(v_cache), _code(k_cache),
               _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1],
               {"none": 0, "plain": 1, "weighted": 2}[norm], _ptr(q_norm_w), _ptr(k_norm_w), float(eps), float(temp_coef),
-              int(temp_every), n, n_q, n_kv, d, dv, k_cache.shape[2], int(write_kv), _stream()), "head_prepare")
+              int(temp_every), n, n_q, n_kv, d, dv, k_cache.shape[2], int(write_kv), _ptr(q_head_scale),
+              -1.0 if v_norm_eps is None else float(v_norm_eps), _stream()), "head_prepare")
     return q_out
 
 
 def paged_attention_wide(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                          positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
-                         n_q: int, n_kv: int, d: int, dv: int, scale: float, window: int = 0) -> torch.Tensor:
+                         n_q: int, n_kv: int, d: int, dv: int, scale: float, window: int = 0, softcap: float = 0.0) -> torch.Tensor:
     """The generic attention kernel with values of their own width: keys of up to 1,024 numbers, values of `dv`.
-    `v_cache` may be `k_cache` itself: a value is then the first dv numbers of its key's row."""
+    `v_cache` may be `k_cache` itself: a value is then the first dv numbers of its key's row.  `softcap` c > 0: a
+    scaled score s becomes c tanh(s / c)."""
     _dev(q, k_cache, v_cache, out, positions, seq_of_token, block_table)
     for t, name in ((positions, "positions"), (seq_of_token, "seq_of_token"), (block_table, "block_table")):
         _i32(t, name)
@@ -446,12 +454,13 @@ def paged_attention_wide(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.
           "attention: caches must be [pages, n_kv, page, d] and [pages, n_kv, page, >= dv] of one type")
     _need(positions.numel() == n and seq_of_token.numel() == n and block_table.dim() == 2,
           "attention: one position and sequence per token, block_table [sequences, blocks]")
-    fn = _fn("attention_generic", "kipp_paged_attention_generic_v",
+    _need(softcap >= 0, "attention: softcap must not be negative")
+    fn = _fn("attention_generic", "kipp_paged_attention_generic_capped",
              [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
-              _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr])
+              _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_float, _c_ptr])
     _check(fn(_ptr(q), _code(q), _ptr(k_cache), _ptr(v_cache), _code(k_cache), _ptr(out), _code(out),
               _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1],
-              n, n_q, n_kv, d, dv, v_cache.shape[3], k_cache.shape[2], float(scale), int(window), _stream()),
+              n, n_q, n_kv, d, dv, v_cache.shape[3], k_cache.shape[2], float(scale), int(window), float(softcap), _stream()),
            "paged_attention_wide")
     return out
 
@@ -578,6 +587,207 @@ def mlstm_finish(o_raw: torch.Tensor, proj: torch.Tensor, gate_at: int, norm_w: 
     fn = _fn("mlstm", "kipp_mlstm_finish", [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_float, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(o_raw), _ptr(proj), proj.shape[1], int(gate_at), _ptr(norm_w), float(eps), _ptr(out), _code(out), n, heads, dv,
               _stream()), "mlstm_finish")
+    return out
+
+
+# --------------------------------------------------------------------------- layer norm and the sandwich step
+
+LAYER_NORM_MAX_WIDTH = 8192
+
+
+def layer_norm(u: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float, out: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """out = scale * ((u - mean) / sqrt(var + eps) * weight + bias) over rows; `u` is float32 [rows, width] or slabs
+    [parts, rows, width] that are added in order."""
+    _dev(u, weight, bias, out)
+    parts, rows, width = _slabs(u, "layer_norm")
+    _need(weight.dtype == bias.dtype == torch.float32 and weight.numel() == bias.numel() == width, "layer_norm: float32 weight and bias [width]")
+    _need(out.shape == (rows, width) and width <= LAYER_NORM_MAX_WIDTH, "layer_norm: out is [rows, width], width up to 8,192")
+    fn = _fn("layer_norm", "kipp_layer_norm", [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_float, _c_ptr, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(u), parts, _ptr(weight), _ptr(bias), float(eps), float(scale), _ptr(out), _code(out), rows, width, _stream()), "layer_norm")
+    return out
+
+
+def sandwich_step(x: torch.Tensor, delta: torch.Tensor, post_w: torch.Tensor, post_b: torch.Tensor, post_eps: float, mult: float,
+                  extra: Optional[torch.Tensor] = None, next_w: Optional[torch.Tensor] = None, next_b: Optional[torch.Tensor] = None,
+                  next_eps: float = 0.0, out: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """x += mult * LN_post(delta) [+ extra] in place (float32 [rows, width]; `delta` may come in slabs), and, with `out`,
+    out = LN_next(x) in out's type: the end of one normed sublayer and the beginning of the next in one pass over a row."""
+    _dev(x, delta, post_w, post_b, extra, next_w, next_b, out)
+    parts, rows, width = _slabs(delta, "sandwich_step")
+    _need(x.dtype == torch.float32 and x.shape == (rows, width) and width <= LAYER_NORM_MAX_WIDTH, "sandwich_step: x is float32 [rows, width], width up to 8,192")
+    for t in (post_w, post_b, next_w, next_b):
+        _need(t is None or (t.dtype == torch.float32 and t.numel() == width), "sandwich_step: float32 weights and biases [width]")
+    _need(extra is None or (extra.dtype == torch.float32 and extra.shape == x.shape), "sandwich_step: extra is float32 of x's shape")
+    _need(out is None or (out.shape == x.shape and next_w is not None and next_b is not None), "sandwich_step: out needs the next norm")
+    fn = _fn("layer_norm", "kipp_sandwich_step", [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_float,
+                                                  _c_ptr, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(x), _ptr(delta), parts, _ptr(post_w), _ptr(post_b), float(post_eps), float(mult), _ptr(extra), _ptr(next_w), _ptr(next_b),
+              float(next_eps), _ptr(out), _code(out) if out is not None else F32, rows, width, _stream()), "sandwich_step")
+    return out
+
+
+# --------------------------------------------------------------------------- matrix memories: fixed decay, gated delta rule
+
+def _scan_args(state, q_start, q_len, slots, o_raw, tokens, heads, d, dv, what):
+    for t, name in ((q_start, "q_start"), (q_len, "q_len"), (slots, "slots")):
+        _i32(t, name)
+    _need(state.dim() == 2 and state.dtype == torch.float32 and state.shape[1] >= heads * d * dv, f"{what}: state is float32 [slots, >= heads d dv]")
+    _need(o_raw.dtype == torch.float32 and o_raw.shape == (tokens, heads * dv) and 0 < d <= 1024, f"{what}: o_raw is float32 [tokens, heads dv]; key size up to 1,024")
+    _need(q_start.numel() == q_len.numel() == slots.numel(), f"{what}: one start, length and slot an entry")
+
+
+def decay_scan(proj: torch.Tensor, decays: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
+               slots: torch.Tensor, o_raw: torch.Tensor, heads: int, d: int, dv: int) -> torch.Tensor:
+    """Linear attention with a fixed decay a head over every entry's tokens, in order, from and into the entry's slot of
+    `state` [slots, size] (float32, S as [head][column][row]).  `proj`: float32 [tokens, >= 2 heads d + heads dv], columns
+    q | k | v before their silu; `o_raw` float32 [tokens, heads dv] receives S^T q."""
+    _dev(proj, decays, state, q_start, q_len, slots, o_raw)
+    _need(proj.dim() == 2 and proj.dtype == torch.float32 and proj.shape[1] >= 2 * heads * d + heads * dv, "decay_scan: proj is float32 [tokens, q | k | v ...]")
+    _need(decays.dtype == torch.float32 and decays.numel() == heads, "decay_scan: float32 decays [heads]")
+    _scan_args(state, q_start, q_len, slots, o_raw, proj.shape[0], heads, d, dv, "decay_scan")
+    fn = _fn("linear_scan", "kipp_decay_scan", [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_size, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(proj), proj.shape[1], _ptr(decays), _ptr(state), state.shape[1], _ptr(q_start), _ptr(q_len), _ptr(slots), _ptr(o_raw),
+              q_start.numel(), heads, d, dv, _stream()), "decay_scan")
+    return o_raw
+
+
+def delta_state_size(heads: int, kv_heads: int, d: int, dv: int, taps: int) -> int:
+    """float32 numbers of a request's state: S [heads, dv, d], then the last taps - 1 inputs of the q | k | v channels."""
+    size = heads * d * dv + (taps - 1) * (2 * kv_heads * d + heads * dv)
+    return -(-size // 4) * 4
+
+
+def delta_prepare(proj: torch.Tensor, conv_w: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor, state: torch.Tensor,
+                  seq_of_token: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor, slots: torch.Tensor, prep: torch.Tensor,
+                  heads: int, kv_heads: int, d: int, dv: int, beta_col: int, a_col: int, unit_eps: float) -> torch.Tensor:
+    """The gated delta rule's inputs from its input product `proj` (float32 [tokens, >= channels], columns q | k | v first,
+    the beta and decay pre-activations at `beta_col` and `a_col`): `prep` [tokens, channels + 2 heads] receives q | k | v
+    behind their short convolutions (`conv_w` [channels, taps], the slot's kept inputs in front of a portion) and silu, every
+    q and k head a unit vector (q also over sqrt(d)), then beta = sigmoid and g = exp(-exp(a_log) softplus(. + dt_bias)) a
+    head.  The slot's kept inputs are then moved on by the portion."""
+    _dev(proj, conv_w, a_log, dt_bias, state, seq_of_token, q_start, q_len, slots, prep)
+    for t, name in ((seq_of_token, "seq_of_token"), (q_start, "q_start"), (q_len, "q_len"), (slots, "slots")):
+        _i32(t, name)
+    channels = 2 * kv_heads * d + heads * dv
+    n = proj.shape[0]
+    _need(proj.dim() == 2 and proj.dtype == torch.float32 and proj.shape[1] >= max(channels, beta_col + heads, a_col + heads), "delta_prepare: proj is float32 [tokens, q | k | v | ...]")
+    _need(conv_w.dtype == torch.float32 and conv_w.dim() == 2 and conv_w.shape[0] == channels and 1 <= conv_w.shape[1] <= 16, "delta_prepare: float32 filters [channels, taps], up to 16 taps")
+    taps = conv_w.shape[1]
+    _need(a_log.dtype == dt_bias.dtype == torch.float32 and a_log.numel() == dt_bias.numel() == heads, "delta_prepare: float32 a_log and dt_bias [heads]")
+    _need(prep.dtype == torch.float32 and prep.shape == (n, channels + 2 * heads) and seq_of_token.numel() == n, "delta_prepare: prep is float32 [tokens, channels + 2 heads]")
+    _need(state.dim() == 2 and state.dtype == torch.float32 and state.shape[1] >= delta_state_size(heads, kv_heads, d, dv, taps), "delta_prepare: state is float32 [slots, size]")
+    _need(q_start.numel() == q_len.numel() == slots.numel(), "delta_prepare: one start, length and slot an entry")
+    fn = _fn("linear_scan", "kipp_delta_prepare", [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_size, _c_size, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                                                   _c_ptr, _c_int] + [_c_int] * 8 + [_c_float, _c_ptr])
+    _check(fn(_ptr(proj), proj.shape[1], _ptr(conv_w), taps, _ptr(a_log), _ptr(dt_bias), _ptr(state), state.shape[1], heads * d * dv,
+              _ptr(seq_of_token), _ptr(q_start), _ptr(q_len), _ptr(slots), _ptr(prep), prep.shape[1], n, q_start.numel(), heads, kv_heads, d, dv,
+              int(beta_col), int(a_col), float(unit_eps), _stream()), "delta_prepare")
+    return prep
+
+
+def delta_scan(prep: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor, slots: torch.Tensor,
+               o_raw: torch.Tensor, heads: int, kv_heads: int, d: int, dv: int) -> torch.Tensor:
+    """The gated delta rule over every entry's tokens, in order, from and into the entry's slot: S <- g S; u = beta (v - S^T k);
+    S <- S + k u^T; o = S^T q, with `prep` as `delta_prepare` leaves it."""
+    _dev(prep, state, q_start, q_len, slots, o_raw)
+    _need(prep.dim() == 2 and prep.dtype == torch.float32 and prep.shape[1] >= 2 * kv_heads * d + heads * dv + 2 * heads and heads % kv_heads == 0,
+          "delta_scan: prep is float32 [tokens, q | k | v | beta | g]")
+    _scan_args(state, q_start, q_len, slots, o_raw, prep.shape[0], heads, d, dv, "delta_scan")
+    fn = _fn("linear_scan", "kipp_delta_scan", [_c_ptr, _c_int, _c_ptr, _c_size, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(prep), prep.shape[1], _ptr(state), state.shape[1], _ptr(q_start), _ptr(q_len), _ptr(slots), _ptr(o_raw), q_start.numel(),
+              heads, kv_heads, d, dv, _stream()), "delta_scan")
+    return o_raw
+
+
+def scan_finish(o_raw: torch.Tensor, gates: torch.Tensor, gate_at: int, norm_w: torch.Tensor, eps: float, gate: str, span: int,
+                out: torch.Tensor) -> torch.Tensor:
+    """out [tokens, width] = every run of `span` columns of `o_raw` over its root mean square, times norm_w[column % len(norm_w)],
+    times gate(gates[:, gate_at + column]), gate "sigmoid" or "silu"."""
+    _dev(o_raw, gates, norm_w, out)
+    n, width = o_raw.shape
+    _need(o_raw.dtype == gates.dtype == norm_w.dtype == torch.float32 and out.shape == o_raw.shape and gates.dim() == 2 and gates.shape[0] == n
+          and gates.shape[1] >= gate_at + width and width % span == 0 and gate in ("sigmoid", "silu"), "scan_finish: float32 rows, gate columns inside `gates`")
+    fn = _fn("linear_scan", "kipp_scan_finish", [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_float, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(o_raw), _ptr(gates), gates.shape[1], int(gate_at), _ptr(norm_w), norm_w.numel(), float(eps), 0 if gate == "sigmoid" else 1,
+              _ptr(out), _code(out), n, width, int(span), _stream()), "scan_finish")
+    return out
+
+
+# --------------------------------------------------------------------------- routed feed-forward
+
+ACTIVATIONS = {"silu": 0, "relu": 1, "gelu": 2, "gelu_tanh": 3}
+MOE_TILE_ROWS = 16
+
+
+def moe_max_tiles(tokens: int, experts: int, top: int) -> int:
+    """Tiles of up to 16 rows that the sorted pairs of a step can need at most (every expert may end in a partial one)."""
+    pairs = tokens * top
+    return -(-pairs // MOE_TILE_ROWS) + min(experts, pairs)
+
+
+def moe_route(z: torch.Tensor, experts: int, top: int, eps: float, chosen: torch.Tensor, weight: torch.Tensor,
+              pair_token: torch.Tensor, place_of_pair: torch.Tensor, tiles: torch.Tensor):
+    """From router logits `z` (float32 [tokens, >= experts] or slabs): softmax over the experts, the `top` largest a token
+    (`chosen`, int32 [tokens, top]) with weights p / (sum of the chosen p + eps) (`weight`, float32 [tokens, top]); then the
+    pairs sorted by expert: `pair_token` [pairs] the token of every sorted row, `place_of_pair` [pairs] the row of pair
+    (token, choice), `tiles` int32 [max_tiles, 3] = (expert, first row, rows), unused tiles with 0 rows."""
+    _dev(z, chosen, weight, pair_token, place_of_pair, tiles)
+    parts, n, stride = _slabs(z, "moe_route")
+    for t, name in ((chosen, "chosen"), (pair_token, "pair_token"), (place_of_pair, "place_of_pair"), (tiles, "tiles")):
+        _i32(t, name)
+    _need(0 < top <= experts <= 1024 and top <= 32 and stride >= experts, "moe_route: up to 1,024 experts, up to 32 a token")
+    _need(chosen.shape == (n, top) and weight.shape == (n, top) and weight.dtype == torch.float32 and pair_token.numel() == n * top
+          and place_of_pair.numel() == n * top and tiles.dim() == 2 and tiles.shape[1] == 3 and tiles.shape[0] >= moe_max_tiles(n, experts, top),
+          "moe_route: output shapes")
+    fn = _fn("moe", "kipp_moe_route", [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr])
+    _check(fn(_ptr(z), parts, stride, _ptr(chosen), _ptr(weight), n, experts, top, float(eps), _ptr(pair_token), _ptr(place_of_pair), _ptr(tiles),
+              tiles.shape[0], _stream()), "moe_route")
+    return chosen, weight
+
+
+def moe_expert(x: torch.Tensor, gather: Optional[torch.Tensor], w: torch.Tensor, tiles: torch.Tensor, out: torch.Tensor,
+               activation: Optional[str] = None) -> torch.Tensor:
+    """Every tile's rows against its expert's matrix: out[row] = act(w[expert] x_row), x_row = x[gather[row]] (or x[row]);
+    `w` [experts, n_out, k], `out` [sorted rows, n_out]."""
+    _dev(x, gather, w, tiles, out)
+    _i32(tiles, "tiles")
+    if gather is not None:
+        _i32(gather, "gather")
+    _need(w.dim() == 3 and x.dim() == 2 and x.shape[1] == w.shape[2] and out.dim() == 2 and out.shape[1] == w.shape[1] and x.dtype == w.dtype,
+          "moe_expert: x [rows, k], w [experts, n_out, k] of one type, out [rows, n_out]")
+    _need(out.shape[0] == (gather.numel() if gather is not None else x.shape[0]), "moe_expert: one output row a sorted row")
+    _need(activation is None or activation in ACTIVATIONS, f"moe_expert: activation is one of {sorted(ACTIVATIONS)}")
+    fn = _fn("moe", "kipp_moe_expert", [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(x), _code(x), _ptr(gather), _ptr(w), _code(w), _ptr(tiles), tiles.shape[0], _ptr(out), _code(out), w.shape[1], w.shape[2],
+              -1 if activation is None else ACTIVATIONS[activation], _stream()), "moe_expert")
+    return out
+
+
+def moe_combine(y: torch.Tensor, place_of_pair: torch.Tensor, weight: torch.Tensor, shared: Optional[torch.Tensor], out: torch.Tensor) -> torch.Tensor:
+    """out[t] = sum_j weight[t, j] y[place_of_pair[t top + j]] + shared[t] (float32; `shared` may come in slabs or be None)."""
+    _dev(y, place_of_pair, weight, shared, out)
+    _i32(place_of_pair, "place_of_pair")
+    n, width = out.shape
+    top = weight.shape[1]
+    _need(y.dtype == weight.dtype == out.dtype == torch.float32 and y.shape == (n * top, width) and place_of_pair.numel() == n * top,
+          "moe_combine: float32 y [tokens top, width], weight [tokens, top], out [tokens, width]")
+    parts = 0
+    if shared is not None:
+        parts, rows, w2 = _slabs(shared, "moe_combine")
+        _need((rows, w2) == (n, width), "moe_combine: shared is [tokens, width] or slabs of it")
+    fn = _fn("moe", "kipp_moe_combine", [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(y), _ptr(place_of_pair), _ptr(weight), _ptr(shared), parts, _ptr(out), n, width, top, _stream()), "moe_combine")
+    return out
+
+
+def activate(u: torch.Tensor, out: torch.Tensor, activation: str, glu: bool = False) -> torch.Tensor:
+    """out = act(u), or with `glu` out[r, i] = act(u[r, i]) * u[r, inner + i]; `u` float32 [rows, width] or slabs of it."""
+    _dev(u, out)
+    parts, rows, width = _slabs(u, "activate")
+    inner = out.shape[1]
+    _need(out.shape[0] == rows and width == (2 * inner if glu else inner) and activation in ACTIVATIONS, "activate: shapes or activation")
+    fn = _fn("moe", "kipp_activate", [_c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(u), parts, _ptr(out), _code(out), rows, inner, int(glu), ACTIVATIONS[activation], _stream()), "activate")
     return out
 
 

@@ -60,6 +60,7 @@ class Model:
         self.final_norm = build_part("norm", spec.final_norm, runtime)
         self.head = build_part("head", spec.head, runtime)
         self.loaded = False
+        self.residual_probe = None      # a callable (run index, float32 residual stream) called after every run, for inspection
 
     # -- what the cache manager has to provide, per run of the order -----------------
     def kv_needs(self):
@@ -115,13 +116,28 @@ class Model:
         if self.input_position is not None:
             x = self.input_position.forward(x, batch)
         pending = None
+        ops = self.rt.ops
+        # the embedding's output, kept for the runs in front of which it is added once more
+        first = ops.copy(x, self.rt.empty(x.shape, x.dtype)) if any(run.add_embedding for run in self.spec.order) else None
         for index, run in enumerate(self.spec.order):
             block = self.blocks[run.layer]
             view = cache.view(index, run.cache_of)
+            if run.add_embedding:
+                if hasattr(pending, "also_add"):
+                    pending = pending.also_add(first)       # the norm that carries the pending delta out adds this as well
+                else:
+                    if pending is not None:
+                        ops.residual_add(x, self.rt.settle(pending))
+                        pending = None
+                    ops.residual_add(x, first)
             x, pending = block.forward(x, pending, batch, view, cache.state(index))
+            if self.residual_probe is not None:
+                if pending is not None:
+                    ops.residual_add(x, self.rt.settle(pending))
+                    pending = None
+                self.residual_probe(index, x)
         if batch.n_want == 0:
             return None
-        ops = self.rt.ops
         if pending is not None and not (batch.want_every_row and getattr(self.final_norm, "fuses_products", False)):
             pending = self.rt.settle(pending)
         if batch.want_every_row:

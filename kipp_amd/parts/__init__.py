@@ -1,5 +1,5 @@
 """The parts a layer is put together from, each chosen by the `kind` of its spec."""
 from .base import (CATEGORIES, ParamSpec, build_part, part_class, part_params,
                    register, unregister)
-from . import (norm, position, mixer, mixed_attention, latent_attention, mlstm, feed_forward, block, streams,  # noqa: F401  (register the parts)
+from . import (norm, position, mixer, mixed_attention, latent_attention, mlstm, matrix_memory, feed_forward, block, streams,  # noqa: F401  (register the parts)
                embedding)

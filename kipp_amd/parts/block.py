@@ -94,3 +94,43 @@ class PostNormMixerBlock(PostNormBlock):
     """The first half of the post-norm arrangement alone: a layer without a feed-forward."""
 
     roles = (("mixer_norm", "norm"), ("mixer", "mixer"))
+
+
+@register("block", "sandwich_norm")
+class SandwichNormBlock:
+    """A norm in front of a sublayer and another on its result: x += a mixer_post_norm(mixer(mixer_norm(x)));
+    x += a ffn_post_norm(ffn(ffn_norm(x))), a = the layer's `residual_scale`.  A sublayer's result is handed on as a
+    `NormedDelta`: the norm in front of the next sublayer (this block's or the next one's) norms it, adds it and norms
+    the new residual in one kernel."""
+
+    roles = (("mixer_norm", "norm"), ("mixer", "mixer"), ("mixer_post_norm", "norm"),
+             ("ffn_norm", "norm"), ("ffn", "feed_forward"), ("ffn_post_norm", "norm"))
+
+    def __init__(self, layer_spec, runtime):
+        self.rt = runtime
+        self.alpha = float(layer_spec.residual_scale)
+        self.parts = {role: build_part(cat, layer_spec.part(role), runtime) for role, cat in self.roles}
+        self.mixer = self.parts["mixer"]
+        self.graph_safe = all(getattr(part, "graph_safe", False) for part in self.parts.values())
+
+    def _sublayer(self, x, pending, norm, post_norm, run):
+        from .norm import NormedDelta
+        rt, act = self.rt, self.rt.act_dtype
+        if pending is not None and not getattr(norm, "fuses_products", False):
+            pending = rt.settle(pending)
+        h = rt.rows_of(norm.forward(x, act) if pending is None else norm.add_forward(x, pending, act))
+        return NormedDelta(rt, rt.settle(run(h)), post_norm, self.alpha)
+
+    def forward(self, x, pending, batch, cache, state):
+        p = self.parts
+        pending = self._sublayer(x, pending, p["mixer_norm"], p["mixer_post_norm"], lambda h: self.mixer.forward(h, batch, cache, state))
+        if "ffn" in p:
+            pending = self._sublayer(x, pending, p["ffn_norm"], p["ffn_post_norm"], lambda h: p["ffn"].forward(h, batch))
+        return x, pending
+
+
+@register("block", "sandwich_norm_mixer")
+class SandwichNormMixerBlock(SandwichNormBlock):
+    """The first half of the sandwich arrangement alone: a layer without a feed-forward."""
+
+    roles = (("mixer_norm", "norm"), ("mixer", "mixer"), ("mixer_post_norm", "norm"))

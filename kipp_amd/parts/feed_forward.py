@@ -12,7 +12,7 @@ from __future__ import annotations
 
 import torch
 
-from ..runtime import ScaledRows
+from ..runtime import ScaledRows, Weight
 from .base import ParamSpec, register
 
 
@@ -42,7 +42,7 @@ class GatedMLP:
         g, u = tensors[gate], tensors[up]
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
-        self.w_gate_up = self.rt.weight(torch.cat([g, u], dim=0).contiguous(), gate_up=True)
+        self.w_gate_up = self.rt.weight(torch.cat([g, u], dim=0).contiguous(), gate_up=self.spec.activation == "silu")
         self.w_down = self.rt.weight(tensors[down])
 
     def forward(self, x, batch=None):
@@ -50,6 +50,11 @@ class GatedMLP:
         rows, inner = x.shape[0], self.spec.intermediate_size
         act = rt.empty((rows, inner), rt.act_dtype)
         w = self.w_gate_up
+        if self.spec.activation != "silu":
+            # another activation: the gate-up product by itself, then the activation's own kernel (the products that
+            # end in the activation are built for silu)
+            rt.ops.activate(rt.linear(rt.rows_of(x), Weight(w.rows, None if w.pairs else w.tiles), slabs=True), act, self.spec.activation, glu=True)
+            return rt.linear(act, self.w_down, slabs=True, defer=True)
         ours = w.dtype == x.dtype == torch.bfloat16 and rt.streams(rows, x.shape[1], 2 * inner)
         if ours and rows <= rt.few_rows:
             # both products and the activation in one kernel (and the norm's scale, if it was left to us)
@@ -72,3 +77,75 @@ class GatedMLP:
         else:
             rt.ops.swiglu(rt.linear(x, w, slabs=True), act)
         return rt.linear(act, self.w_down, slabs=True, defer=True)
+
+
+@register("feed_forward", "routed_mlp")
+class RoutedMLP:
+    """A mixture of experts (`RoutedMLPSpec`): delta = sum over a token's `top` experts of weight_e W_down_e act(W_up_e x),
+    plus a shared expert of the same form.  The router's logits come out of a product in float32; choice, sort and the
+    experts' products over the sorted rows are kernels whose launches have a fixed shape (the list of row tiles is made on
+    the device), so nothing is read back and a step of single tokens can be recorded."""
+
+    graph_safe = True   # forward launches kernels only: no host reads, no data-dependent launches
+
+    def __init__(self, spec, runtime):
+        self.spec = spec
+        self.rt = runtime
+        self.w_router = self.w_up = self.w_down = self.w_shared_up = self.w_shared_down = None
+
+    @staticmethod
+    def params(spec):
+        s = spec
+        up, down = s.names
+        p = {s.router_name: ParamSpec((s.experts, s.hidden_size))}
+        for e in range(s.experts):
+            p[s.expert_prefix.format(e) + up] = ParamSpec((s.expert_size, s.hidden_size))
+            p[s.expert_prefix.format(e) + down] = ParamSpec((s.hidden_size, s.expert_size))
+        if s.shared_size is not None:
+            p[s.shared_prefix + up] = ParamSpec((s.shared_size, s.hidden_size))
+            p[s.shared_prefix + down] = ParamSpec((s.hidden_size, s.shared_size))
+        return p
+
+    @staticmethod
+    def variants(spec, dtype):
+        return [("moe", None)]
+
+    def load(self, tensors):
+        s = self.spec
+        up, down = s.names
+        router = tensors[s.router_name]
+        pad = -router.shape[0] % 16     # whole tiles of rows for the products
+        if pad:
+            router = torch.cat([router, torch.zeros((pad, router.shape[1]), dtype=router.dtype, device=router.device)], dim=0)
+        self.w_router = self.rt.weight(router.contiguous())
+        ups = [tensors[s.expert_prefix.format(e) + up] for e in range(s.experts)]
+        downs = [tensors[s.expert_prefix.format(e) + down] for e in range(s.experts)]
+        if len({t.dtype for t in ups + downs}) > 1:
+            ups, downs = [t.float() for t in ups], [t.float() for t in downs]
+        self.w_up = torch.stack(ups).contiguous()           # [experts, inner, hidden]
+        self.w_down = torch.stack(downs).contiguous()       # [experts, hidden, inner]
+        if s.shared_size is not None:
+            self.w_shared_up = self.rt.weight(tensors[s.shared_prefix + up])
+            self.w_shared_down = self.rt.weight(tensors[s.shared_prefix + down])
+
+    def forward(self, x, batch=None):
+        s, rt, ops = self.spec, self.rt, self.rt.ops
+        n = x.shape[0]
+        pairs = n * s.top
+        dev = rt.device
+        z = rt.linear(x, self.w_router, slabs=True)
+        chosen = torch.empty((n, s.top), dtype=torch.int32, device=dev)
+        weight = rt.empty((n, s.top), torch.float32)
+        pair_token = torch.empty((pairs,), dtype=torch.int32, device=dev)
+        place = torch.empty((pairs,), dtype=torch.int32, device=dev)
+        tiles = torch.empty((ops.moe_max_tiles(n, s.experts, s.top), 3), dtype=torch.int32, device=dev)
+        ops.moe_route(z, s.experts, s.top, s.weight_eps, chosen, weight, pair_token, place, tiles)
+        if x.dtype != self.w_up.dtype:
+            x = ops.cast(x, rt.empty(x.shape, self.w_up.dtype))
+        inner = ops.moe_expert(x, pair_token, self.w_up, tiles, rt.empty((pairs, s.expert_size), self.w_up.dtype), s.activation)
+        y = ops.moe_expert(inner, None, self.w_down, tiles, rt.empty((pairs, s.hidden_size), torch.float32))
+        shared = None
+        if s.shared_size is not None:
+            mid = ops.activate(rt.linear(x, self.w_shared_up, slabs=True), rt.empty((n, s.shared_size), rt.act_dtype), s.activation)
+            shared = rt.linear(mid, self.w_shared_down, slabs=True)
+        return ops.moe_combine(y, place, weight, shared, rt.empty((n, s.hidden_size), torch.float32))

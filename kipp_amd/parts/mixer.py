@@ -55,12 +55,14 @@ class Attention:
         if spec.qk_norm_eps is not None and spec.qk_norm_weight:
             p[q_norm] = ParamSpec((spec.head_dim,), "float", ("one_plus_normal", 0.05))
             p[k_norm] = ParamSpec((spec.head_dim,), "float", ("one_plus_normal", 0.05))
+        if spec.head_temp is not None:
+            p[spec.head_temp] = ParamSpec((spec.num_heads,), "float", ("one_plus_normal", 0.2))
         return p
 
     @staticmethod
     def placement(spec):
         """What enters norms and sums in float32 is widened on the device (exact)."""
-        return {name: "float32" for name in spec.names[4:] + tuple(spec.bias_names)}
+        return {name: "float32" for name in spec.names[4:] + tuple(spec.bias_names) + ((spec.head_temp,) if spec.head_temp else ())}
 
     @staticmethod
     def variants(spec, dtype):
@@ -68,7 +70,7 @@ class Attention:
         that share a key/value head).  Under float32, and for more than 16 heads a group, the generic
         attention kernel runs, which every model has."""
         out = [("rope_kv", None) if spec.plain else ("head_prepare", None), ("attention_generic", None)]
-        if dtype != "bfloat16" or spec.head_dim % 16 or spec.value_dim != spec.head_dim:
+        if dtype != "bfloat16" or spec.head_dim % 16 or spec.value_dim != spec.head_dim or spec.softcap is not None:
             return out
         group = spec.num_heads // spec.num_kv_heads
         out.append(("attention_prefill", {"HEAD_DIM": spec.head_dim}))
@@ -89,6 +91,7 @@ class Attention:
         if s.qk_norm_eps is not None and s.qk_norm_weight:
             self.q_norm = tensors[names[4]]
             self.k_norm = tensors[names[5]]
+        self.head_temp = tensors[s.head_temp] if s.head_temp is not None else None
         self.bias = None
         if s.bias:
             held = [tensors[name] for name in (s.bias_names if s.own_kv else s.bias_names[:1])]
@@ -178,23 +181,23 @@ class Attention:
         q = rt.ops.head_prepare(proj, rt.empty((n, s.q_dim), rt.act_dtype), cache.k, cache.v, batch.positions,
                                 batch.seq_of_token, table, s.num_heads, s.num_kv_heads, d, dv, self.bias, norm,
                                 s.qk_norm_eps or 0.0, self.q_norm, self.k_norm, coef, every,
-                                write_kv=cache.writable and s.own_kv)
-        fast = rt.dtype == "bfloat16" and d % 16 == 0 and d == dv \
+                                write_kv=cache.writable and s.own_kv, q_head_scale=self.head_temp, v_norm_eps=s.v_norm_eps)
+        fast = rt.dtype == "bfloat16" and d % 16 == 0 and d == dv and s.softcap is None \
             and rt.ops.attention_fast_ok(s.num_heads, s.num_kv_heads, cache.page_size, table.shape[1])
         if rt.dtype == "bfloat16" and not fast:
             rt.generic_attention_launches += 1
         out = rt.empty((n, s.out_dim), rt.act_dtype)
         paged_attention(rt, batch, q, out, cache.k, cache.v, cache.page_size, table, s.num_heads, s.num_kv_heads, d, dv,
-                        self.scale, s.window, fast, owner=self)
+                        self.scale, s.window, fast, owner=self, softcap=s.softcap or 0.0)
         return rt.linear(out, self.w_o, slabs=True, defer=True)
 
 
-def paged_attention(rt, batch, q, out, k_cache, v_cache, page_size, table, n_q, n_kv, d, dv, scale, window, fast, owner=None):
+def paged_attention(rt, batch, q, out, k_cache, v_cache, page_size, table, n_q, n_kv, d, dv, scale, window, fast, owner=None, softcap=0.0):
     """The attention itself over a paged cache, for any mixer that has its queries ready: q [tokens, n_q d] -> out
     [tokens, n_q dv].  `fast`: the matrix-core kernels (prompt portions and single tokens each by their own; they
     need d == dv, or `v_cache` being `k_cache`, a value then being as wide as its key's row); else the generic kernel,
     which takes values of their own width (`v_cache` may be `k_cache` there too: a value is the first dv numbers
-    of its key's row).  `owner`: a mixer whose `_prefill_work(batch)` and `_workspace(batch)` make the work list and the
+    of its key's row).  `softcap` c > 0: a scaled score s becomes c tanh(s / c) (the generic kernel).  `owner`: a mixer whose `_prefill_work(batch)` and `_workspace(batch)` make the work list and the
     decode workspace (else they are made here for these sizes)."""
     if fast:
         if batch.n_portions:
@@ -205,13 +208,13 @@ def paged_attention(rt, batch, q, out, k_cache, v_cache, page_size, table, n_q, 
             rt.ops.attention_decode(q, k_cache, v_cache, out, batch.decode_rows, batch.positions, batch.seq_of_token, table,
                                     n_q, n_kv, d, scale, window or 0, batch.max_decode_ctx,
                                     owner._workspace(batch) if owner is not None else decode_workspace(rt, batch, n_q, d))
-    elif d == dv and v_cache is not k_cache and d <= 256:
+    elif d == dv and v_cache is not k_cache and d <= 256 and not softcap:
         # the float32 path, and geometries the matrix-core kernels refuse (groups above 16, odd page sizes)
         rt.ops.paged_attention_generic(q, k_cache, v_cache, out, batch.positions, batch.seq_of_token, table, n_q, n_kv, d,
                                        scale, window or 0)
     else:
         rt.ops.paged_attention_wide(q, k_cache, v_cache, out, batch.positions, batch.seq_of_token, table, n_q, n_kv, d, dv,
-                                    scale, window or 0)
+                                    scale, window or 0, softcap=softcap)
     return out
 
 

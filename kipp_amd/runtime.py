@@ -78,7 +78,16 @@ class ScaledRows:
         return self.rows.dtype
 
 
-class Deferred:
+class Pending:
+    """A delta of the residual stream that is not a tensor yet: `run()` makes the float32 tensor (or its slabs).  A norm
+    that knows a kind of pending delta may carry it out together with its own work; everybody else asks `Runtime.settle`."""
+    __slots__ = ()
+
+    def run(self) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Deferred(Pending):
     """A product `x . w^T` that `Runtime.linear(..., defer=True)` has not launched
     yet: the delta of a mixer or a feed-forward, which a norm that follows may
     launch together with the residual add (`Runtime.product_add_norm`); `run()`
@@ -168,7 +177,7 @@ class Runtime:
 
     def settle(self, delta):
         """The tensor of a delta, launched now if it was deferred."""
-        return delta.run() if isinstance(delta, Deferred) else delta
+        return delta.run() if isinstance(delta, Pending) else delta
 
     def rows_of(self, h):
         """The tensor of norm output, scaled now if the scale was left to a product."""
