@@ -43,7 +43,7 @@ class BebulornConfig:
 
     @classmethod
     def from_dict(cls, d: dict) -> "BebulornConfig":
-        _only(d, ("architecture", "architectures", "vocab", "width", "norm", "residual_mult", "layers", "loop", "max_position"), "")
+        _only(d, ("architecture", "architectures", "vocab", "width", "norm", "residual_mult", "layers", "loop", "max_position", "torch_dtype"), "")
         layers = _get(d, "layers", "")
         if not isinstance(layers, list) or not layers:
             raise ConfigError("config.json layers: expected a list with at least one layer")

@@ -1,0 +1,571 @@
+"""The Bebulorn design on the GPU against its plain implementation: every new kernel alone (crafted inputs at the edges),
+then the engine under every cutting in both precisions, tight pools, slots used again, long decoding, recorded steps,
+other sizes, generation through the scheduler, the trace replay and the command line."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from tests import helpers as H
+from tests.plain import bebulorn_plain as P
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SHAPES = ("bebulorn-tiny-a", "bebulorn-tiny-b")
+LENGTHS = [1, 19, 45, 80, 131]
+TOL = {"float32": 1e-9, "bfloat16": 3e-2}     # float32 is the sharp test; at these narrow widths bfloat16 rows are noisy and a close call of a router may fall the other way
+
+
+def sharpen(folder, factor=10.0):
+    """Larger query and key matrices in the attention layers, so that few keys carry a row's softmax and a key that is
+    wrongly seen or missed shows in the logits."""
+    from safetensors import safe_open
+    from safetensors.torch import save_file
+    path = os.path.join(folder, "model.safetensors")
+    with open(os.path.join(folder, "config.json")) as f:
+        cfg = json.load(f)
+    tensors = {}
+    with safe_open(path, framework="pt") as f:
+        for name in f.keys():
+            tensors[name] = f.get_tensor(name)
+    for i, layer in enumerate(cfg["layers"]):
+        if layer["type"] == "attention":
+            for which in ("q", "k"):
+                tensors[f"l{i}.mix.{which}"] = (tensors[f"l{i}.mix.{which}"].float() * factor).to(tensors[f"l{i}.mix.{which}"].dtype)
+    save_file(tensors, path)
+    return folder
+
+
+def write_model(path, cfg, seed, dtype):
+    from kipp_amd.weights import write_random_model
+    return sharpen(write_random_model(str(path), cfg, seed=seed, dtype=dtype))
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    from kipp_amd.config import shape_config
+    root = tmp_path_factory.mktemp("bebulorn")
+    return {(shape, dtype): write_model(root / f"{shape}-{dtype}", shape_config(shape), 40 + i, dtype)
+            for i, shape in enumerate(SHAPES) for dtype in ("float32", "bfloat16")}
+
+
+_plain_cache = {}
+
+
+def plain_logits(folder, tokens):
+    key = (folder, tuple(tokens))
+    if key not in _plain_cache:
+        cfg, w = P.load_folder(folder)
+        _plain_cache[key] = P.forward_whole(cfg, w, list(tokens))
+    return _plain_cache[key]
+
+
+FLIPS = 0.5       # share of a request's positions that may lie beyond the bfloat16 bound (see `close`)
+
+
+def close(got, ref, tol, what):
+    """Every position's normalised squared error within `tol`.  Under the bfloat16 bound a share of the positions may lie
+    beyond it: a router's choice between two experts whose scores differ by less than the rounding of the rows it reads
+    falls either way, and the position (and, through memories that forget slowly or never, every one after it) then
+    differs by much more than rounding.  The float32 runs of the same cases allow no such position; what is wrong for most positions (a window, a
+    state, a page) fails either bound."""
+    assert got.shape == ref.shape and np.isfinite(got).all(), what
+    errs = sorted(float(np.sum((g - r) ** 2) / np.sum(r ** 2)) for g, r in zip(got.astype(np.float64), ref))
+    spared = int(FLIPS * len(errs)) if tol >= TOL["bfloat16"] else 0
+    worst = errs[len(errs) - 1 - spared]
+    over = sum(e > tol for e in errs)
+    assert worst <= tol, f"{what}: NMSE {worst:.3e} exceeds {tol:.1e} ({over} of {len(errs)} positions beyond it, {spared} spared)"
+
+
+def engine_of(folder, dtype, page=16, **kw):
+    from kipp_amd.engine import Engine
+    kw.setdefault("max_tokens", 1024)
+    return Engine.from_folder(folder, dtype=dtype, page_size=page, share_prefixes=False, **kw)
+
+
+def dev(a, ty=None):
+    import torch
+    return None if a is None else torch.tensor(np.asarray(a), device="cuda:0", dtype=ty)
+
+
+def f32(a):
+    import torch
+    return dev(np.asarray(a, dtype=np.float32), torch.float32)
+
+
+def i32(a):
+    import torch
+    return dev(np.asarray(a, dtype=np.int32), torch.int32)
+
+
+def bf16(x):
+    import torch
+    return torch.tensor(np.asarray(x, dtype=np.float32)).bfloat16().float().numpy().astype(np.float64)
+
+
+def requests_of(vocab, seed=0, lengths=LENGTHS):
+    return {f"r{i}": H.random_tokens(seed * 100 + i, n, vocab) for i, n in enumerate(lengths)}
+
+
+# =============================================================================== the kernels alone
+
+@pytest.mark.parametrize("width", [40, 256, 1000, 2304])
+def test_layer_norm_and_the_step_between_sublayers(width):
+    import torch
+    from kipp_amd.csrc import ops
+    rng = np.random.default_rng(width)
+    n = 5
+    x, delta, extra = rng.normal(size=(n, width)) * 3 + 1, rng.normal(size=(3, n, width)), rng.normal(size=(n, width))
+    w1, b1, w2, b2 = (rng.normal(size=width) for _ in range(4))
+    ref = P.layer_norm(np.float32(delta).astype(np.float64).sum(axis=0), np.float32(w1), np.float32(b1), 1e-5)
+    got = ops.layer_norm(f32(delta), f32(w1), f32(b1), 1e-5, torch.empty((n, width), device="cuda:0"), scale=0.7)
+    assert np.allclose(got.cpu().numpy(), 0.7 * ref, atol=2e-5)
+    for with_extra in (False, True):
+        xd = f32(x)
+        out = ops.sandwich_step(xd, f32(delta), f32(w1), f32(b1), 1e-5, 0.7, f32(extra) if with_extra else None, f32(w2), f32(b2), 1e-6,
+                                torch.empty((n, width), device="cuda:0"))
+        new_x = np.float32(x).astype(np.float64) + 0.7 * ref + (np.float32(extra) if with_extra else 0.0)
+        assert np.allclose(xd.cpu().numpy(), new_x, atol=3e-5)
+        assert np.allclose(out.cpu().numpy(), P.layer_norm(new_x, np.float32(w2), np.float32(b2), 1e-6), atol=5e-5)
+    xd = f32(x)
+    assert ops.sandwich_step(xd, f32(delta[0]), f32(w1), f32(b1), 1e-5, 1.0) is None       # the add alone
+    assert np.allclose(xd.cpu().numpy(), np.float32(x) + P.layer_norm(np.float32(delta[0]), np.float32(w1), np.float32(b1), 1e-5), atol=3e-5)
+    out16 = ops.layer_norm(f32(delta[1]), f32(w1), f32(b1), 1e-5, torch.empty((n, width), device="cuda:0", dtype=torch.bfloat16))
+    assert np.allclose(out16.float().cpu().numpy(), P.layer_norm(np.float32(delta[1]), np.float32(w1), np.float32(b1), 1e-5), rtol=1e-2, atol=1e-2)
+
+
+def _entries(lengths, slots):
+    starts = np.concatenate([[0], np.cumsum(lengths)[:-1]])
+    seq_of = np.concatenate([np.full(n, i) for i, n in enumerate(lengths)])
+    return i32(starts), i32(lengths), i32(slots), i32(seq_of), starts
+
+
+@pytest.mark.parametrize("heads, d, dv", [(4, 32, 64), (3, 20, 72), (1, 128, 130), (2, 300, 24), (5, 3, 1), (1, 600, 40), (2, 64, 300)])
+def test_decay_scan_over_entries_with_kept_states(heads, d, dv):
+    """Three entries of unequal length in slots of any order, then their next tokens (portions and single tokens) from the
+    kept states: both launches against the plain walk over the whole sequences."""
+    import torch
+    from kipp_amd.csrc import ops
+    rng = np.random.default_rng(heads * 1000 + d)
+    decay = rng.uniform(0.5, 1.0, size=heads).astype(np.float32)
+    decay[0] = 1.0
+    totals, first = [23, 7, 40], [17, 6, 1]
+    width = 2 * heads * d + heads * dv + 5
+    seqs = [rng.normal(size=(t, width)).astype(np.float32) for t in totals]
+    size = -(-heads * d * dv // 4) * 4
+    state = torch.zeros((6, size), device="cuda:0")
+    slots = [4, 0, 2]
+    got = [[] for _ in totals]
+    for part in (0, 1, 2):
+        lengths = [first[i] if part == 0 else (1 if part == 1 else totals[i] - first[i] - 1) for i in range(3)]
+        at = [0 if part == 0 else (first[i] if part == 1 else first[i] + 1) for i in range(3)]
+        live = [i for i in range(3) if lengths[i] > 0]
+        proj = np.concatenate([seqs[i][at[i]:at[i] + lengths[i]] for i in live])
+        qs, ql, sl, _, starts = _entries([lengths[i] for i in live], [slots[i] for i in live])
+        o = ops.decay_scan(f32(proj), f32(decay), state, qs, ql, sl, torch.empty((proj.shape[0], heads * dv), device="cuda:0"), heads, d, dv)
+        o = o.cpu().numpy()
+        for j, i in enumerate(live):
+            got[i].append(o[starts[j]:starts[j] + lengths[i]])
+    for i, t in enumerate(totals):
+        s = seqs[i].astype(np.float64)
+        q = P.silu(s[:, :heads * d]).reshape(t, heads, d)
+        k = P.silu(s[:, heads * d:2 * heads * d]).reshape(t, heads, d)
+        v = P.silu(s[:, 2 * heads * d:2 * heads * d + heads * dv]).reshape(t, heads, dv)
+        ref, S = P.lightning_scan(q, k, v, decay.astype(np.float64))
+        out = np.concatenate(got[i]).reshape(t, heads, dv)
+        assert np.allclose(out, ref, rtol=2e-4, atol=2e-4 * np.abs(ref).max()), (i, np.abs(out - ref).max())
+        kept = state[slots[i], :heads * d * dv].cpu().numpy().reshape(heads, dv, d)
+        assert np.allclose(kept, S.transpose(0, 2, 1), rtol=2e-4, atol=2e-4 * np.abs(S).max())
+    assert float(state[[1, 3, 5]].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("heads, groups, d, dv, taps", [(4, 2, 16, 24, 3), (6, 3, 64, 32, 4), (2, 2, 36, 20, 2), (3, 1, 130, 8, 1), (2, 1, 600, 16, 5), (1, 1, 8, 260, 16)])
+def test_delta_rule_kernels_across_cuts(heads, groups, d, dv, taps):
+    """Filters, unit norms, gates and the recurrence over portions of 1, 2 and more tokens, shorter and longer than the
+    filter, from states kept in slots: against the plain mixer pieces over the whole sequences."""
+    import torch
+    from kipp_amd.csrc import ops
+    rng = np.random.default_rng(heads * 100 + d + taps)
+    channels = 2 * groups * d + heads * dv
+    hv = heads * dv
+    width = channels + hv + 2 * heads + 3
+    beta_col, a_col = channels + hv, channels + hv + heads
+    conv = rng.normal(size=(channels, taps)).astype(np.float32)
+    a_log, dt = rng.normal(size=heads).astype(np.float32) * 0.5, rng.normal(size=heads).astype(np.float32)
+    totals = [31, 12]
+    seqs = [rng.normal(size=(t, width)).astype(np.float32) * 2 for t in totals]
+    cuts = [[5, 1, 1, 2, 9, 1, 12], [1, 1, 2, 3, 1, 1, 3]]
+    state = torch.zeros((4, ops.delta_state_size(heads, groups, d, dv, taps)), device="cuda:0")
+    slots = [3, 1]
+    got = [[], []]
+    at = [0, 0]
+    for step in range(7):
+        lengths = [cuts[i][step] for i in range(2)]
+        proj = np.concatenate([seqs[i][at[i]:at[i] + lengths[i]] for i in range(2)])
+        qs, ql, sl, seq_of, starts = _entries(lengths, slots)
+        n = proj.shape[0]
+        pd = f32(proj)
+        prep = ops.delta_prepare(pd, f32(conv), f32(a_log), f32(dt), state, seq_of, qs, ql, sl, torch.empty((n, channels + 2 * heads), device="cuda:0"),
+                                 heads, groups, d, dv, beta_col, a_col, 1e-6)
+        o = ops.delta_scan(prep, state, qs, ql, sl, torch.empty((n, hv), device="cuda:0"), heads, groups, d, dv).cpu().numpy()
+        for i in range(2):
+            got[i].append(o[starts[i]:starts[i] + lengths[i]])
+            at[i] += lengths[i]
+    for i, t in enumerate(totals):
+        s = seqs[i].astype(np.float64)
+        y = P.silu(P.short_conv(s[:, :channels], conv))
+        q = P.unit(y[:, :groups * d].reshape(t, groups, d)) * d ** -0.5
+        k = P.unit(y[:, groups * d:2 * groups * d].reshape(t, groups, d))
+        v = y[:, 2 * groups * d:].reshape(t, heads, dv)
+        rep = heads // groups
+        beta = P.sigmoid(s[:, beta_col:beta_col + heads])
+        g = np.exp(-np.exp(a_log.astype(np.float64)) * P.softplus(s[:, a_col:a_col + heads] + dt))
+        ref, S = P.delta_scan(np.repeat(q, rep, axis=1), np.repeat(k, rep, axis=1), v, beta, g)
+        out = np.concatenate(got[i]).reshape(t, heads, dv)
+        assert np.allclose(out, ref, rtol=3e-4, atol=3e-4 * np.abs(ref).max()), (i, np.abs(out - ref).max())
+        kept = state[slots[i], :heads * d * dv].cpu().numpy().reshape(heads, dv, d)
+        assert np.allclose(kept, S.transpose(0, 2, 1), rtol=3e-4, atol=3e-4 * max(np.abs(S).max(), 1e-6))
+        if taps > 1:
+            last = state[slots[i], heads * d * dv:heads * d * dv + (taps - 1) * channels].cpu().numpy().reshape(taps - 1, channels)
+            want = np.concatenate([np.zeros((max(0, taps - 1 - t), channels)), seqs[i][max(0, t - (taps - 1)):, :channels]])
+            assert np.array_equal(last, want.astype(np.float32))
+
+
+@pytest.mark.parametrize("gate, span, w_len", [("sigmoid", 96, 96), ("silu", 24, 24), ("silu", 1, 1), ("sigmoid", 600, 600)])
+def test_scan_finish(gate, span, w_len):
+    import torch
+    from kipp_amd.csrc import ops
+    rng = np.random.default_rng(span)
+    n, width = 6, span * 4 if span < 600 else 600
+    o, gates, w = rng.normal(size=(n, width)), rng.normal(size=(n, width + 9)), rng.normal(size=w_len)
+    got = ops.scan_finish(f32(o), f32(gates), 7, f32(w), 1e-5, gate, span, torch.empty((n, width), device="cuda:0")).cpu().numpy()
+    o32 = np.float32(o).astype(np.float64)
+    normed = P.rms(o32.reshape(n, width // span, span), 1e-5).reshape(n, width) * np.tile(np.float32(w), width // w_len)
+    z = np.float32(gates[:, 7:7 + width]).astype(np.float64)
+    ref = normed * (P.sigmoid(z) if gate == "sigmoid" else P.silu(z))
+    assert np.allclose(got, ref, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("experts, top, tokens, width, inner", [(16, 2, 37, 64, 96), (5, 3, 1, 72, 40), (8, 1, 300, 40, 24), (70, 4, 129, 32, 520), (3, 3, 20, 300, 16)])
+def test_routed_feed_forward_kernels(dtype, experts, top, tokens, width, inner):
+    """Choice and weights (with logits that tie), the sort into runs of one expert (some experts get nothing, some more than
+    a tile), both expert products and the weighted sum with a shared part in slabs: against loops over tokens."""
+    import torch
+    from kipp_amd.csrc import ops
+    rng = np.random.default_rng(experts * 10 + top)
+    ty = torch.float32 if dtype == "float32" else torch.bfloat16
+    rnd = (lambda a: np.float32(a).astype(np.float64)) if dtype == "float32" else bf16
+    z = rng.normal(size=(2, tokens, experts + 3)).astype(np.float32) * 2
+    z[:, :, experts // 2] = -30.0              # an expert that nobody takes
+    if tokens > 2:
+        z[:, 2, :] = 0.0                        # every score equal: the lowest indices
+    x = rnd(rng.normal(size=(tokens, width)))
+    w_up, w_down = rnd(rng.normal(size=(experts, inner, width)) * 0.2), rnd(rng.normal(size=(experts, width, inner)) * 0.2)
+    shared = rng.normal(size=(2, tokens, width)).astype(np.float32)
+    pairs = tokens * top
+    chosen, weight = torch.empty((tokens, top), dtype=torch.int32, device="cuda:0"), torch.empty((tokens, top), device="cuda:0")
+    pair_token, place = torch.empty(pairs, dtype=torch.int32, device="cuda:0"), torch.empty(pairs, dtype=torch.int32, device="cuda:0")
+    tiles = torch.full((ops.moe_max_tiles(tokens, experts, top), 3), -7, dtype=torch.int32, device="cuda:0")
+    ops.moe_route(f32(z), experts, top, 1e-20, chosen, weight, pair_token, place, tiles)
+    zz = z.astype(np.float64).sum(axis=0)[:, :experts]
+    e = np.exp(zz - zz.max(axis=1, keepdims=True))
+    s = e / e.sum(axis=1, keepdims=True)
+    ref_chosen = np.argsort(-s, axis=1, kind="stable")[:, :top]
+    picked = np.take_along_axis(s, ref_chosen, axis=1)
+    ref_weight = picked / (picked.sum(axis=1, keepdims=True) + 1e-20)
+    if tokens > 2:
+        assert chosen[2].tolist() == list(range(top))
+    got_chosen = chosen.cpu().numpy()
+    assert np.array_equal(np.sort(got_chosen, axis=1), np.sort(ref_chosen, axis=1))
+    order = np.argsort(got_chosen, axis=1), np.argsort(ref_chosen, axis=1)
+    assert np.allclose(np.take_along_axis(weight.cpu().numpy(), order[0], axis=1), np.take_along_axis(ref_weight, order[1], axis=1), rtol=1e-4, atol=1e-6)
+    # the sort: a permutation, every tile within one expert's run
+    pl, pt, tl = place.cpu().numpy(), pair_token.cpu().numpy(), tiles.cpu().numpy()
+    assert sorted(pl.tolist()) == list(range(pairs)) and np.array_equal(pt[pl], np.arange(pairs) // top)
+    expert_of_row = np.empty(pairs, dtype=np.int64)
+    expert_of_row[pl] = got_chosen.reshape(-1)
+    assert np.all(np.diff(expert_of_row) >= 0)
+    covered = np.zeros(pairs, dtype=int)
+    for ex, first, rows in tl:
+        assert 0 <= rows <= 16
+        if rows:
+            assert np.all(expert_of_row[first:first + rows] == ex)
+            covered[first:first + rows] += 1
+    assert np.all(covered == 1)
+    mid = ops.moe_expert(dev(x, ty), pair_token, dev(w_up, ty), tiles, torch.empty((pairs, inner), dtype=ty, device="cuda:0"), "gelu")
+    y = ops.moe_expert(mid, None, dev(w_down, ty), tiles, torch.empty((pairs, width), device="cuda:0"))
+    out = ops.moe_combine(y, place, weight, f32(shared), torch.empty((tokens, width), device="cuda:0")).cpu().numpy()
+    ref = shared.astype(np.float64).sum(axis=0)
+    wt = weight.cpu().numpy().astype(np.float64)
+    for t in range(tokens):
+        for j in range(top):
+            ex = got_chosen[t, j]
+            m = P.gelu_erf(x[t] @ w_up[ex].T)
+            ref[t] += wt[t, j] * ((m if dtype == "float32" else bf16(m)) @ w_down[ex].T)
+    tol = 1e-4 if dtype == "float32" else 2e-2
+    assert np.allclose(out, ref, rtol=tol, atol=tol * np.abs(ref).max()), np.abs(out - ref).max()
+    # the activations' own kernel: a gated and a plain one, from slabs
+    u = rng.normal(size=(2, 7, 2 * inner)).astype(np.float32)
+    us = u.astype(np.float64).sum(axis=0)
+    glu = ops.activate(f32(u), torch.empty((7, inner), device="cuda:0"), "relu", glu=True).cpu().numpy()
+    assert np.allclose(glu, np.maximum(us[:, :inner], 0) * us[:, inner:], rtol=1e-5, atol=1e-6)
+    assert np.allclose(ops.activate(f32(u), torch.empty((7, 2 * inner), device="cuda:0"), "gelu").cpu().numpy(), P.gelu_erf(us), rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H_, G, d, dv, window, page", [(4, 2, 32, 32, 40, 16), (6, 2, 24, 16, 11, 8), (3, 3, 96, 96, 17, 16), (2, 1, 80, 200, 64, 32), (2, 2, 16, 16, None, 16)])
+def test_capped_attention_with_a_key_that_stands_out(dtype, H_, G, d, dv, window, page):
+    """Head factors, value norm and the cap against the plain attention on random inputs; then one key whose score stands out
+    far back, at a page border, just inside and just outside the window: seen by the last row of a prompt portion and by
+    a single token exactly when the design says so."""
+    import torch
+    from kipp_amd.csrc import ops
+    ty = torch.float32 if dtype == "float32" else torch.bfloat16
+    rng = np.random.default_rng(d + (window or 0))
+    T, scale, cap, eps = 150, 0.3, 6.0, 1e-5
+    temp = rng.uniform(0.5, 2.0, size=H_).astype(np.float32)
+    pages = -(-T // page)
+    order = rng.permutation(pages + 3)[:pages]
+    table = i32(order.reshape(1, pages))
+    positions, seq_of = i32(np.arange(T)), i32(np.zeros(T))
+
+    def run(proj, rows):
+        kc = torch.zeros((pages + 3, G, page, d), dtype=ty, device="cuda:0")
+        vc = torch.zeros((pages + 3, G, page, dv), dtype=ty, device="cuda:0")
+        q = ops.head_prepare(f32(proj), torch.empty((T, H_ * d), dtype=ty, device="cuda:0"), kc, vc, positions, seq_of, table, H_, G, d, dv, None,
+                             "none", 0.0, q_head_scale=f32(temp), v_norm_eps=eps)
+        idx = np.asarray(rows)
+        out = torch.empty((len(idx), H_ * dv), dtype=ty, device="cuda:0")
+        ops.paged_attention_wide(q[dev(idx, torch.int64)].contiguous(), kc, vc, out, i32(idx), i32(np.zeros(len(idx))), table, H_, G, d, dv, scale,
+                                 window or 0, softcap=cap)
+        return out.float().cpu().numpy().reshape(len(idx), H_, dv)
+
+    proj = rng.normal(size=(T, H_ * d + G * d + G * dv)).astype(np.float32)
+    p64 = proj.astype(np.float64)
+    q, k = p64[:, :H_ * d].reshape(T, H_, d), p64[:, H_ * d:H_ * d + G * d].reshape(T, G, d)
+    v = P.rms(p64[:, H_ * d + G * d:].reshape(T, G, dv), eps)
+    ref = P.capped_attention(q, k, v, G, scale, temp.astype(np.float64), cap, window)
+    tol = 1e-4 if dtype == "float32" else 6e-2
+    assert np.allclose(run(proj, range(T)), ref, rtol=tol, atol=tol)
+    # one key stands out: every other score is near -cap, its own near +cap
+    u = rng.normal(size=d).astype(np.float32)
+    u /= np.linalg.norm(u)
+    last = T - 1
+    w = window if window is not None else T
+    for key, seen in ((last - w + 1, True), (last - w, False), (0, window is None), (-(-(last - w + 1) // page) * page, True), (last, True)):
+        if key < 0 or (not seen and window is None):
+            continue
+        crafted = proj.copy()
+        crafted[:, H_ * d:H_ * d + G * d] = np.tile(-100.0 * u, G)
+        crafted[last, :H_ * d] = np.tile(u, H_)
+        crafted[key, H_ * d:H_ * d + G * d] = np.tile(100.0 * u, G)
+        mark = np.zeros(dv, dtype=np.float32)
+        mark[0] = 1.0
+        crafted[key, H_ * d + G * d:] = np.tile(50.0 * mark, G)          # after its norm: sqrt(dv) in the first place
+        for rows in (range(T), [last]):
+            got = run(crafted, rows)[-1]
+            if seen:
+                assert np.allclose(got[:, 0], np.sqrt(dv), rtol=2e-2), (key, list(rows)[:2], got[:, 0])
+            else:
+                assert np.all(np.abs(got[:, 0]) < 0.9 * np.sqrt(dv)), (key, list(rows)[:2], got[:, 0])
+
+
+# =============================================================================== the engine
+
+@pytest.mark.parametrize("dtype, page", [("float32", 16), ("bfloat16", 16), ("bfloat16", 32), ("float32", 8)])
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("cut", ["whole", "tail", "portions", "mixed"])
+def test_cuttings_match_plain(folders, shape, dtype, page, cut):
+    """Whole prompts, the last tokens one by one, portions of changing size down to two tokens, and mixed batches in a
+    pool that only holds the live requests and has four state slots (pages and slots are used again)."""
+    folder = folders[(shape, dtype)]
+    vocab = P.load_folder(folder)[0]["vocab"]
+    requests = requests_of(vocab)
+    if cut == "mixed":
+        requests.update({f"s{i}": H.random_tokens(900 + i, n, vocab) for i, n in enumerate(LENGTHS)})
+        steps = H.mixed(requests, seed=5)
+        engine = engine_of(folder, dtype, page, max_tokens=None, num_pages=H.peak_pages(requests, steps, page), max_requests=4)
+    else:
+        engine = engine_of(folder, dtype, page)
+        steps = {"whole": H.whole, "tail": H.tail_one_by_one, "portions": H.changing_portions}[cut](requests)
+    got = H.replay(engine, requests, steps)
+    for rid, toks in requests.items():
+        close(got[rid], plain_logits(folder, toks), TOL[dtype], f"{shape}/{dtype}/{page}/{cut}/{rid}")
+    assert engine.cache.free_pages() == [g.pool.num_pages for g in engine.cache.groups]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_float32_cuttings_are_bitwise_equal(folders, shape):
+    """In float32 every sum runs in an order that the token's own position fixes: how the prompt was cut, what else was
+    in the batch and which pages and slots were used change no bit."""
+    folder = folders[(shape, "float32")]
+    requests = requests_of(P.load_folder(folder)[0]["vocab"], seed=3)
+    base = H.replay(engine_of(folder, "float32"), requests, H.whole(requests))
+    for maker in (H.tail_one_by_one, H.changing_portions, lambda r: H.mixed(r, seed=11)):
+        steps = maker(requests)
+        order = list(np.random.default_rng(1).permutation(64))
+        got = H.replay(engine_of(folder, "float32", page_order=order, max_requests=5), requests, steps)
+        for rid in requests:
+            assert np.array_equal(got[rid], base[rid]), f"{shape}/{rid}: bits differ between cuttings"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_through_a_small_pool_and_one_slot(tmp_path, dtype):
+    """A window of 20 in pages of 16 beside both memories, the loop run twice: 200 tokens pass through the few pages that
+    the window needs and the one state slot, which a second request then takes over (its memories and its filters' last
+    inputs must start at zero, not where the first left them)."""
+    cfg = {"architecture": "Bebulorn", "vocab": 90, "width": 64, "norm": {"eps": 1e-5}, "residual_mult": 0.8,
+           "loop": {"start": 0, "stop": 3, "times": 2},
+           "layers": [{"type": "attention", "mixer": {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 16, "scale": 0.25, "softcap": 10.0, "mask": {"size": 20}},
+                       "mlp": {"kind": "dense", "ff": 48}},
+                      {"type": "delta", "mixer": {"heads": 2, "kv_heads": 1, "dim": 16, "vdim": 24, "conv": 4}, "mlp": None},
+                      {"type": "lightning", "mixer": {"heads": 2, "dim": 16, "vdim": 16, "decay": [0.8, 0.99]},
+                       "mlp": {"kind": "moe", "router": {"experts": 4, "top": 2}, "expert": {"ff": 32}, "shared": {"ff": 32}}}]}
+    folder = write_model(tmp_path / "three", cfg, 8, dtype)
+    tokens = {"r": H.random_tokens(77, 200, 90), "next": H.random_tokens(78, 40, 90)}
+    engine = engine_of(folder, dtype, 16, max_tokens=None, num_pages=4, max_requests=1)
+    steps = [([("r", 10)], [])] + [([("r", 1)], []) for _ in range(60)] + [([("r", 7)], []), ([("r", 2)], [])] \
+        + [([("r", 1)], []) for _ in range(121)]
+    steps[-1] = (steps[-1][0], ["r"])
+    steps += [([("next", 33)], [])] + [([("next", 1)], []) for _ in range(7)]
+    steps[-1] = (steps[-1][0], ["next"])
+    got = H.replay(engine, tokens, steps)
+    for rid in tokens:
+        close(got[rid], plain_logits(folder, tokens[rid]), TOL[dtype], f"four pages/{dtype}/{rid}")
+    if dtype == "bfloat16":
+        assert engine.graphs.replays > 100          # the single tokens ran as recorded steps
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_other_sizes_and_branches(tmp_path, dtype):
+    """Widths that are no multiple of 8 or of 32, a window of one, no window and no cap (the matrix-core attention under
+    bfloat16), eighteen heads on one key/value head, memories with keys wider than 256, one tap, one expert of one, a
+    loop over the last layers only, a loop that runs once; prompts of more rows than the few-rows products take."""
+    layers = [
+        {"type": "attention", "mixer": {"heads": 18, "kv_heads": 1, "dim": 16, "vdim": 16, "scale": 0.3, "mask": {"size": 1}}, "mlp": None},
+        {"type": "lightning", "mixer": {"heads": 1, "dim": 260, "vdim": 20, "decay": [0.9]}, "mlp": {"kind": "dense", "ff": 30}},
+        {"type": "attention", "mixer": {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 32, "scale": 0.2}, "mlp": {"kind": "moe", "router": {"experts": 1, "top": 1}, "expert": {"ff": 20}}},
+        {"type": "delta", "mixer": {"heads": 3, "kv_heads": 3, "dim": 264, "vdim": 12, "conv": 1}, "mlp": {"kind": "dense", "ff": 52}},
+        {"type": "attention", "mixer": {"heads": 3, "kv_heads": 3, "dim": 40, "vdim": 24, "scale": 0.1, "softcap": 2.0, "mask": {"size": 300}},
+         "mlp": {"kind": "moe", "router": {"experts": 9, "top": 9}, "expert": {"ff": 8}, "shared": {"ff": 100}}}]
+    for width, loop in ((100, {"start": 3, "stop": 5, "times": 2}), (72, {"start": 1, "stop": 2, "times": 1})):
+        cfg = {"architecture": "Bebulorn", "vocab": 77, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 1.0, "loop": loop, "layers": layers}
+        folder = write_model(tmp_path / f"odd{width}", cfg, width, dtype)
+        requests = {"long": H.random_tokens(1, 330, 77), "short": H.random_tokens(2, 9, 77)}
+        for steps in (H.whole(requests), [([("long", 270)], []), ([("long", 59), ("short", 8)], []), ([("long", 1), ("short", 1)], ["long", "short"])]):
+            got = H.replay(engine_of(folder, dtype), requests, steps)
+            for rid, toks in requests.items():
+                close(got[rid], plain_logits(folder, toks), TOL[dtype] * (4 if dtype == "bfloat16" else 1), f"{width}/{dtype}/{rid}")
+
+
+def random_configuration(rng):
+    """A model of the design with every size, the order of its layers and every constant drawn at random."""
+    layers = []
+    for i in range(rng.randint(3, 6)):
+        kind = rng.choice(["attention", "lightning", "delta"])
+        r = rng.random()
+        if r < 0.15:
+            mlp = None
+        elif r < 0.55:
+            mlp = {"kind": "dense", "ff": rng.choice([128, 200, 384])}
+        else:
+            experts = rng.choice([2, 4, 7, 16])
+            mlp = {"kind": "moe", "router": {"experts": experts, "top": rng.randint(1, min(4, experts))}, "expert": {"ff": rng.choice([24, 64, 100])}}
+            if rng.random() < 0.6:
+                mlp["shared"] = {"ff": rng.choice([32, 72])}
+        if kind == "attention":
+            groups = rng.choice([1, 2, 3, 4])
+            d = rng.choice([16, 32, 40, 64, 96])
+            mixer = {"heads": groups * rng.choice([1, 2, 3]), "kv_heads": groups, "dim": d, "vdim": d if rng.random() < 0.5 else rng.choice([16, 24, 64]),
+                     "scale": rng.uniform(0.05, 0.3), "softcap": rng.choice([5.0, 20.0, 50.0]), "mask": {"size": rng.choice([1, 5, 16, 17, 64, 100, 300])}}
+        elif kind == "lightning":
+            heads = rng.choice([1, 2, 4])
+            mixer = {"heads": heads, "dim": rng.choice([16, 48, 64, 160]), "vdim": rng.choice([16, 48, 100]), "decay": [rng.uniform(0.5, 1.0) for _ in range(heads)]}
+        else:
+            groups = rng.choice([1, 2, 3])
+            mixer = {"heads": groups * rng.choice([1, 2]), "kv_heads": groups, "dim": rng.choice([16, 48, 64, 128]), "vdim": rng.choice([16, 32, 80]),
+                     "conv": rng.choice([1, 2, 4, 7])}
+        layers.append({"type": kind, "mixer": mixer, "mlp": mlp})
+    cfg = {"architecture": "Bebulorn", "vocab": rng.choice([300, 512]), "width": rng.choice([96, 128, 192]), "residual_mult": rng.choice([0.3, 1.0, 1.4]),
+           "norm": {"eps": rng.choice([1e-5, 1e-6])}, "layers": layers}
+    if rng.random() < 0.8:
+        start = rng.randint(0, len(layers) - 1)
+        cfg["loop"] = {"start": start, "stop": rng.randint(start + 1, len(layers)), "times": rng.randint(1, 3)}
+    return cfg
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_models_drawn_at_random(tmp_path, seed):
+    """Sizes, order of layers and constants drawn at random; whole prompts, portions and mixed batches in float32."""
+    import random
+    cfg = random_configuration(random.Random(seed))
+    folder = write_model(tmp_path / "drawn", cfg, seed, "float32")
+    requests = {f"r{i}": H.random_tokens(seed * 10 + i, n, cfg["vocab"]) for i, n in enumerate([1, 23, 97, 180])}
+    for maker in (H.whole, H.changing_portions, lambda r: H.mixed(r, seed=seed)):
+        got = H.replay(engine_of(folder, "float32", max_requests=4), requests, maker(requests))
+        for rid, toks in requests.items():
+            close(got[rid], plain_logits(folder, toks), 2e-8, f"drawn {seed}/{rid}: {json.dumps(cfg)}")
+
+
+def test_recorded_steps_of_a_changing_batch(folders):
+    """Three requests decode together from recorded steps while the window passes page borders and the memories go on in
+    their slots; one ends early and the batch goes on at another size."""
+    folder = folders[("bebulorn-tiny-a", "bfloat16")]
+    vocab = P.load_folder(folder)[0]["vocab"]
+    requests = {"a": H.random_tokens(1, 90, vocab), "b": H.random_tokens(2, 120, vocab), "c": H.random_tokens(3, 75, vocab)}
+    engine = engine_of(folder, "bfloat16")
+    steps = [([("a", 30), ("b", 51), ("c", 2)], [])]
+    fed = {"a": 30, "b": 51, "c": 2}
+    while any(fed[r] < len(requests[r]) for r in fed):
+        live = [r for r in fed if fed[r] < len(requests[r])]
+        for r in live:
+            fed[r] += 1
+        steps.append(([(r, 1) for r in live], [r for r in live if fed[r] == len(requests[r])]))
+    got = H.replay(engine, requests, steps)
+    for rid, toks in requests.items():
+        close(got[rid], plain_logits(folder, toks), TOL["bfloat16"], f"recorded/{rid}")
+    assert engine.graphs.replays > 50
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_scheduler(folders, dtype):
+    """`generate` (scheduler, continuous batching, tokens chosen on the device) against the plain implementation:
+    every generated token is the plain argmax of its position, or within rounding of it."""
+    from kipp_amd import generate
+    folder = folders[("bebulorn-tiny-b", dtype)]
+    cfg, w = P.load_folder(folder)
+    prompts = [H.random_tokens(5, 3, cfg["vocab"]), H.random_tokens(6, 40, cfg["vocab"]), H.random_tokens(7, 21, cfg["vocab"])]
+    outputs = generate(folder, prompts, max_new_tokens=30, dtype=dtype, page_size=16, prefill_chunk=16, max_step_tokens=24)
+    margin = 1e-4 if dtype == "float32" else 0.05
+    for prompt, out in zip(prompts, outputs):
+        assert len(out) == 30
+        logits = P.forward_whole(cfg, w, prompt + out)
+        for i, tok in enumerate(out):
+            row = logits[len(prompt) - 1 + i]
+            assert row[tok] >= row.max() - margin * (row.max() - row.min()), (dtype, i)
+
+
+def test_trace_replay_and_command_line(folders, tmp_path):
+    folder = folders[("bebulorn-tiny-a", "bfloat16")]
+    vocab = P.load_folder(folder)[0]["vocab"]
+    toks = H.random_tokens(4, 60, vocab)
+    lines = [{"step": 0, "entries": [{"id": "x", "tokens": toks[:33], "want": [0, 32]}], "end": []},
+             {"step": 1, "entries": [{"id": "x", "tokens": toks[33:35], "want": []}, {"id": "y", "tokens": toks[:7], "want": [6]}], "end": ["y"]},
+             {"step": 2, "entries": [{"id": "x", "tokens": toks[35:36], "want": [0]}], "end": ["x"]}]
+    out = tmp_path / "out"
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", "bfloat16", "--out", str(out),
+                          "--max-tokens", "128"], input="\n".join(json.dumps(l) for l in lines) + "\n", capture_output=True, text=True, timeout=600)
+    assert run.returncode == 0, run.stderr[-2000:]
+    assert [l for l in run.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    ref = plain_logits(folder, toks)
+    close(np.fromfile(out / "0.f32", dtype="<f4").reshape(2, vocab), ref[[0, 32]], TOL["bfloat16"], "trace step 0")
+    close(np.fromfile(out / "1.f32", dtype="<f4").reshape(1, vocab), ref[[6]], TOL["bfloat16"], "trace step 1")
+    close(np.fromfile(out / "2.f32", dtype="<f4").reshape(1, vocab), ref[[35]], TOL["bfloat16"], "trace step 2")
+    cli = subprocess.run([sys.executable, "-m", "kipp_amd.cli", "--model", folder, "--tokens", ",".join(map(str, toks[:9])), "--decode", "5"],
+                         capture_output=True, text=True, timeout=600, cwd=ROOT)
+    assert cli.returncode == 0, cli.stderr[-2000:]
