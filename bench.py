@@ -244,6 +244,9 @@ def long_context_points(model, rt, cfg, numbers, args, weight_bytes, kv_per_toke
     return points, fracs
 
 
+DESIGN_KINDS_DEFAULT = "attention,latent,latent_wide,mlstm,mixed"
+
+
 def tobinex_config(qwen: dict, layers: int, window) -> dict:
     """A Tobinex configuration with the layer sizes of a Qwen3 shape: the same width, heads, head size (keys and values
     alike), feed-forward and vocabulary; `window` None keeps every key, as the Qwen3 layers do."""
@@ -284,6 +287,36 @@ def rerizen_config(qwen: dict, layers: int, kind: str) -> dict:
         made.append({"type": name, "mixer": mixer, "mlp": {"kind": "dense", "ff": qwen["intermediate_size"]}})
     return {"architecture": "Rerizen", "vocab": qwen["vocab_size"], "width": width, "streams": 2, "logit_scale": 1.0,
             "norm": {"eps": 1e-6}, "max_position": 8192, "layers": made}
+
+
+def bebulorn_config(qwen: dict, layers: int, kind: str) -> dict:
+    """A Bebulorn configuration with the layer sizes of a Qwen3 shape (width, feed-forward, vocabulary) and `layers` layers
+    of one kind, so that every mechanism's kernels stand beside their like alone: "attention" (Qwen3's heads and head size,
+    scores capped at 30, a window of 1,024 keys, a factor a head, values normed; dense feed-forward), "lightning" and "delta"
+    (the two matrix memories at the geometry of Rerizen's mLSTM: 8 heads, keys of 128 or 256, values that fill the width;
+    the delta rule with a filter of 4 taps and one query/key head for every two heads), "moe" (the attention mixer with a
+    routed feed-forward: 32 experts of a quarter of the dense inner size, 4 a token, and a shared one as large, so that a
+    token multiplies about as much as in the dense layer), or "mixed" (lightning + dense, attention + routed, delta + dense,
+    lightning + routed, the last three run twice as a loop)."""
+    width, heads = qwen["hidden_size"], qwen["num_attention_heads"]
+    head_dim = qwen.get("head_dim") or width // heads
+    ff = qwen["intermediate_size"]
+    attention = {"heads": heads, "kv_heads": qwen["num_key_value_heads"], "dim": head_dim, "vdim": head_dim, "scale": head_dim ** -0.5,
+                 "softcap": 30.0, "mask": {"size": 1024}}
+    key = 128 if width <= 2560 else 256
+    lightning = {"heads": 8, "dim": key, "vdim": width // 8, "decay": [1.0 - 2.0 ** -(3 + i) for i in range(8)]}
+    delta = {"heads": 8, "kv_heads": 4, "dim": key, "vdim": width // 8, "conv": 4}
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "router": {"experts": 32, "top": 4}, "expert": {"ff": ff // 4}, "shared": {"ff": ff // 4}}
+    kinds = {"attention": [("attention", attention, dense)], "lightning": [("lightning", lightning, dense)],
+             "delta": [("delta", delta, dense)], "moe": [("attention", attention, moe)],
+             "mixed": [("lightning", lightning, dense), ("attention", attention, moe), ("delta", delta, dense), ("lightning", lightning, moe)]}
+    order = kinds[kind]
+    made = [{"type": order[i % len(order)][0], "mixer": dict(order[i % len(order)][1]), "mlp": dict(order[i % len(order)][2])}
+            for i in range(layers)]
+    loop = {"start": 1, "stop": layers, "times": 2} if kind == "mixed" and layers > 1 else {"start": 0, "stop": layers, "times": 1}
+    return {"architecture": "Bebulorn", "vocab": qwen["vocab_size"], "width": width, "norm": {"eps": 1e-5}, "residual_mult": 0.7,
+            "loop": loop, "layers": made}
 
 
 def design_points(config, args, label):
@@ -352,6 +385,27 @@ def rerizen_bench(args) -> int:
     return 0
 
 
+def bebulorn_bench(args) -> int:
+    """`--design bebulorn`: the Bebulorn design beside Qwen3 and beside Rerizen's mLSTM layers (the framework's other matrix
+    memory) at equal layer sizes, a few layers of each, random weights: one model for each of its mechanisms alone, and one
+    with all of them in turn under a loop."""
+    from kipp_amd.config import shape_config
+    layers = args.layers or 4
+    kinds = args.design_kinds if args.design_kinds != DESIGN_KINDS_DEFAULT else "attention,lightning,delta,moe,mixed"
+    sizes = {}
+    for shape in [s for s in args.design_shapes.split(",") if s]:
+        qwen = shape_config(shape)
+        qwen["num_hidden_layers"] = layers
+        sizes[shape] = {"qwen3": design_points(qwen, args, f"{shape} qwen3"),
+                        "rerizen_mlstm": design_points(rerizen_config(qwen, layers, "mlstm"), args, f"{shape} rerizen, mlstm")}
+        for kind in [k for k in kinds.split(",") if k]:
+            sizes[shape][f"bebulorn_{kind}"] = design_points(bebulorn_config(qwen, layers, kind), args, f"{shape} bebulorn, {kind}")
+    print(json.dumps({"metric": "prefill and decode of the Bebulorn design beside Qwen3 and Rerizen's mLSTM at equal layer sizes (bf16, random weights)",
+                      "design": "bebulorn", "layers": layers, "prompt_tokens": args.prompt, "steps": args.steps,
+                      "unit": "ms and tok/s", "n_gpus": 1, "dtype": "bf16", "data": "synthetic", "sizes": sizes}), flush=True)
+    return 0
+
+
 def design_bench(args) -> int:
     """`--design tobinex`: the Tobinex design beside Qwen3 at equal layer sizes (both with every key kept, and Tobinex
     once more with a window of 1,024 keys behind 4 kept ones), a few layers of each, random weights."""
@@ -391,17 +445,20 @@ def main():
     ap.add_argument("--no-c-host", action="store_true", help="leave out the points measured through the C host")
     ap.add_argument("--products", choices=["default", "own", "auto", "library"], default="default",
                     help="products of many rows (prompt portions): the runtime's default, our kernel only, the fastest of ours and the library's, the library's")
-    ap.add_argument("--design", choices=["tobinex", "rerizen"], default=None,
+    ap.add_argument("--design", choices=["tobinex", "rerizen", "bebulorn"], default=None,
                     help="instead of the default workload: this design beside Qwen3 at equal layer sizes (prefill and decode, a few layers)")
     ap.add_argument("--design-shapes", default="qwen3-4b,qwen3-8b", help="the Qwen3 shapes whose layer sizes --design takes")
-    ap.add_argument("--design-kinds", default="attention,latent,latent_wide,mlstm,mixed",
-                    help="--design rerizen: the models that are measured, one mixer each or all in turn")
+    ap.add_argument("--design-kinds", default=DESIGN_KINDS_DEFAULT,
+                    help="--design rerizen or bebulorn: the models that are measured, one mechanism each or all in turn "
+                         "(bebulorn: attention,lightning,delta,moe,mixed)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
     if args.design == "rerizen":
         return rerizen_bench(args)
+    if args.design == "bebulorn":
+        return bebulorn_bench(args)
     if args.design:
         return design_bench(args)
 

@@ -54,6 +54,20 @@
 #error "compile with -DGROUP=<query heads per key/value head>"
 #endif
 
+// SOFTCAP 1: a score s (the product of a query that was already multiplied by scale / cap, and a key) becomes tanh(s),
+// and the `scale` the launcher is given is the cap: weight = exp(cap tanh(q . k scale / cap) - maximum).
+#ifndef SOFTCAP
+#define SOFTCAP 0
+#endif
+#if SOFTCAP
+// 1 - 2 / (1 + e^(2 s)): +-1 at the ends (the exponential overflows to infinity, or is 0), absolute error about 1e-7
+__device__ __forceinline__ float capped_score(float s) {
+    return 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(s * 2.8853900817779268f));
+}
+#else
+__device__ __forceinline__ float capped_score(float s) { return s; }
+#endif
+
 #define SPLIT 256                              // keys of a split (the kernel that takes one a workgroup also has longer ones)
 #define SPLIT_MIN 192                          // the shortest (few sequences)
 #define SPLIT_MAX 320                          // the longest (the fused form has registers for no more with two workgroups a compute unit)
@@ -430,7 +444,7 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
             for (int v = 0; v < 4; ++v) {
                 const int kl = (wave * BPW + b) * 16 + 4 * h + v;
                 const int s = base + kl;
-                s_scores[l16][kl] = (s >= lo && s <= pos) ? acc[v] * scale_log2e : -INFINITY;
+                s_scores[l16][kl] = (s >= lo && s <= pos) ? capped_score(acc[v]) * scale_log2e : -INFINITY;
             }
         }
     }
@@ -636,7 +650,7 @@ __global__ void __launch_bounds__(THREADS) attention_decode_stream_kernel(
                 for (int v = 0; v < 4; ++v) {
                     const int kl = (wave * SUB_BLOCKS_PER_WAVE + b) * 16 + 4 * h + v;
                     const int sk = first + kl;
-                    s_scores[l16][kl] = (sk >= lo && sk <= pos) ? sc[v] * scale_log2e : -INFINITY;
+                    s_scores[l16][kl] = (sk >= lo && sk <= pos) ? capped_score(sc[v]) * scale_log2e : -INFINITY;
                 }
             }
         }
@@ -998,7 +1012,7 @@ __global__ void __launch_bounds__(THREADS, 2) attention_decode_ring_kernel(
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const int s = (kb << 4) + 4 * h + v;
-            sc[v] = (s >= lo && s <= pos) ? __fmul_rn(sc[v], scale_log2e) : -INFINITY;   // every rounding spelt out: both forms of the kernel give the same bits
+            sc[v] = (s >= lo && s <= pos) ? __fmul_rn(capped_score(sc[v]), scale_log2e) : -INFINITY;   // every rounding spelt out: both forms of the kernel give the same bits
             m_blk = fmaxf(m_blk, sc[v]);
         }
         m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 16, KIPP_WAVE));

@@ -31,6 +31,20 @@
 #error "compile with -DHEAD_DIM=<head size>"
 #endif
 
+// SOFTCAP 1: a score s (the product of a query that was already multiplied by scale / cap, and a key) becomes tanh(s),
+// and the `scale` the launcher is given is the cap: weight = exp(cap tanh(q . k scale / cap) - maximum).
+#ifndef SOFTCAP
+#define SOFTCAP 0
+#endif
+#if SOFTCAP
+// 1 - 2 / (1 + e^(2 s)): +-1 at the ends (the exponential overflows to infinity, or is 0), absolute error about 1e-7
+__device__ __forceinline__ float capped_score(float s) {
+    return 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(s * 2.8853900817779268f));
+}
+#else
+__device__ __forceinline__ float capped_score(float s) { return s; }
+#endif
+
 #define BM 128
 #define BN 64
 #define WAVES 4
@@ -213,6 +227,12 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_kernel(
         // ---- online softmax in base 2; register v of half j is key 32 j + 8 (v / 4) + 4 hh + v % 4.
         //      The scale is folded into the exponent: p = 2^(s c - m c), one FMA and one exp a key.
         //      Only tiles that touch the diagonal (or a window's edge) pay for a mask.
+#if SOFTCAP
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) s_acc[j][v] = capped_score(s_acc[j][v]);
+#endif
         const bool masked = key0 + BN - 1 > pos0 + wave * 32 || window > 0;
         if (masked) {
 #pragma unroll
@@ -488,6 +508,12 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_dma_kernel(
         KIPP_K_STEP(7, 0);
 #undef KIPP_K_READ
 #undef KIPP_K_STEP
+#if SOFTCAP
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) s_acc[j][v] = capped_score(s_acc[j][v]);
+#endif
         const bool masked = key0 + BN - 1 > pos0 + wave * 32 || window > 0;
         if (masked) {
 #pragma unroll

@@ -3,10 +3,14 @@
 //
 //     route    p = softmax(z) over all experts (float32); the `top` largest p (the lower index first among equals);
 //              weight = p / (sum of the chosen p + eps)
-//     sort     the (token, choice) pairs in runs of one expert each, cut into tiles of up to 16 rows; the list of tiles
+//     sort     the (token, choice) pairs in runs of one expert each, cut into tiles of up to 16 (or 64) rows; the list of tiles
 //              is made on the device, so the host never learns the counts and the launches have a fixed shape
-//     expert   a tile's rows against its expert's matrix: out[row][n] = act(sum_k W_e[n][k] x[row][k]); a lane takes a
-//              column, the sum over k runs in index order, so a row's result does not depend on its tile
+//     expert   a tile's rows against its expert's matrix: out[row][n] = act(sum_k W_e[n][k] x[row][k]).  bfloat16 with K a
+//              multiple of 32: on the matrix cores, a workgroup a (tile of up to 64 rows, 256 columns), a wave 64 of the
+//              columns in 4 x 4 fragments of 16 x 16, operands straight from memory (a fragment row is 64 bytes of a
+//              matrix row); a tile of a few rows (single tokens) multiplies only the fragments it has, and is then bound
+//              by the read of its expert's matrix.  Else (float32, other K): a lane takes a column of a tile of 16 rows.
+//              Either way the sum over k runs in one order for every row, so a row's result does not depend on its tile
 //     combine  out[t] = sum_j weight[t][j] y[place of (t, j)] (+ the shared expert's result, slabs added in order)
 #include "common.h"
 #include <math.h>
@@ -17,6 +21,9 @@
 #define TILE_ROWS 16
 #define EXPERT_COLS 256
 #define EXPERT_KC 128
+#define MFMA_ROWS 64        // rows of a tile of the matrix-core product: four fragments of 16
+#define MFMA_COLS 256       // columns of a workgroup: four waves with four fragments each
+#define MFMA_THREADS 256
 
 enum { ACT_NONE = -1, ACT_SILU = 0, ACT_RELU = 1, ACT_GELU = 2, ACT_GELU_TANH = 3 };
 
@@ -88,7 +95,7 @@ moe_route_kernel(const float* __restrict__ z, int parts, size_t part_stride, int
 // One workgroup sorts all pairs.  tiles: int32 [max_tiles][3] = (expert, first row, rows); rows 0 marks an unused tile.
 __global__ void __launch_bounds__(1024)
 moe_sort_kernel(const int32_t* __restrict__ chosen, int pairs, int experts, int top, int32_t* __restrict__ pair_token,
-                int32_t* __restrict__ place_of_pair, int32_t* __restrict__ tiles, int max_tiles) {
+                int32_t* __restrict__ place_of_pair, int32_t* __restrict__ tiles, int max_tiles, int tile_rows) {
     __shared__ int count[MAX_EXPERTS];
     __shared__ int first[MAX_EXPERTS + 1];
     __shared__ int tile_first[MAX_EXPERTS + 1];
@@ -102,7 +109,7 @@ moe_sort_kernel(const int32_t* __restrict__ chosen, int pairs, int experts, int 
             first[e] = rows;
             tile_first[e] = tl;
             rows += count[e];
-            tl += (count[e] + TILE_ROWS - 1) / TILE_ROWS;
+            tl += (count[e] + tile_rows - 1) / tile_rows;
         }
         first[experts] = rows;
         tile_first[experts] = tl;
@@ -110,11 +117,11 @@ moe_sort_kernel(const int32_t* __restrict__ chosen, int pairs, int experts, int 
     __syncthreads();
     for (int e = threadIdx.x; e < experts; e += blockDim.x) {
         const int n = count[e];
-        for (int j = 0; j * TILE_ROWS < n; ++j) {
+        for (int j = 0; j * tile_rows < n; ++j) {
             int32_t* tile = tiles + (size_t)(tile_first[e] + j) * 3;
             tile[0] = e;
-            tile[1] = first[e] + j * TILE_ROWS;
-            tile[2] = min(TILE_ROWS, n - j * TILE_ROWS);
+            tile[1] = first[e] + j * tile_rows;
+            tile[2] = min(tile_rows, n - j * tile_rows);
         }
     }
     for (int i = tile_first[experts] + threadIdx.x; i < max_tiles; i += blockDim.x) {
@@ -175,6 +182,91 @@ moe_expert_kernel(const TX* __restrict__ x, const int32_t* __restrict__ gather, 
         if (r < rows) store_f(out + (size_t)(row0 + r) * n_out, col, activate(acc[r], act));
 }
 
+// The same on the matrix cores: bfloat16 x and w, K a multiple of 32, tiles of up to MFMA_ROWS rows.  A 16 x 16 x 32
+// product takes, from lane l, 8 numbers of row l % 16 at k = 8 (l / 16) .. + 7 of either operand, and leaves
+// C[4 (l / 16) + v][l % 16] in its register v.
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+union Frag {
+    u32x4 u;
+    bf16x8 v;
+};
+
+template <typename TO>
+__global__ void __launch_bounds__(MFMA_THREADS)
+moe_expert_mfma_kernel(const bf16_t* __restrict__ x, const int32_t* __restrict__ gather, const bf16_t* __restrict__ w,
+                       const int32_t* __restrict__ tiles, TO* __restrict__ out, int n_out, int k, int act) {
+    const int32_t* tile = tiles + (size_t)blockIdx.x * 3;
+    const int rows = tile[2];
+    if (rows == 0) return;      // uniform over the workgroup
+    const int expert = tile[0], row0 = tile[1];
+    const int wave = threadIdx.x / KIPP_WAVE, lane = threadIdx.x & (KIPP_WAVE - 1), l16 = lane & 15, h = lane >> 4;
+    const int col0 = blockIdx.y * MFMA_COLS + wave * 64;
+    if (col0 >= n_out) return;  // uniform over the wave; the kernel has no barrier
+    const int mfrags = (rows + 15) >> 4;
+    const bf16_t* a_ptr[4];
+    const bf16_t* b_ptr[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = min(16 * i + l16, rows - 1);          // rows beyond the tile's read its last one and are not stored
+        const size_t src = gather != nullptr ? (size_t)gather[row0 + r] : (size_t)(row0 + r);
+        a_ptr[i] = x + src * k + 8 * h;
+        const int c = min(col0 + 16 * i + l16, n_out - 1);
+        b_ptr[i] = w + ((size_t)expert * n_out + c) * k + 8 * h;
+    }
+    f32x4 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+    if (mfrags == 4) {
+#pragma unroll 2
+        for (int k0 = 0; k0 < k; k0 += 32) {
+            Frag a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                a[i].u = *(const u32x4*)(a_ptr[i] + k0);
+                b[i].u = *(const u32x4*)(b_ptr[i] + k0);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i].v, b[j].v, acc[i][j], 0, 0, 0);
+        }
+    } else {
+#pragma unroll 2
+        for (int k0 = 0; k0 < k; k0 += 32) {
+            Frag b[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[j].u = *(const u32x4*)(b_ptr[j] + k0);
+#pragma unroll
+            for (int i = 0; i < 3; ++i) {
+                if (i < mfrags) {
+                    Frag a;
+                    a.u = *(const u32x4*)(a_ptr[i] + k0);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b[j].v, acc[i][j], 0, 0, 0);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int r = 16 * i + 4 * h + v;
+            if (r < rows) {
+                TO* dst = out + (size_t)(row0 + r) * n_out;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int c = col0 + 16 * j + l16;
+                    if (c < n_out) store_f(dst, c, activate(acc[i][j][v], act));
+                }
+            }
+        }
+}
+
 // out[t][c] = sum_j weight[t][j] y[place[t top + j]][c] + sum of the slabs of shared[t][c]
 __global__ void moe_combine_kernel(const float* __restrict__ y, const int32_t* __restrict__ place, const float* __restrict__ weight,
                                    const float* __restrict__ shared, int shared_parts, size_t shared_stride,
@@ -190,22 +282,39 @@ __global__ void moe_combine_kernel(const float* __restrict__ y, const int32_t* _
 }
 
 extern "C" int kipp_moe_route(const float* z, int parts, int stride, int32_t* chosen, float* weight, int tokens, int experts, int top,
-                              float eps, int32_t* pair_token, int32_t* place_of_pair, int32_t* tiles, int max_tiles, hipStream_t stream) {
+                              float eps, int32_t* pair_token, int32_t* place_of_pair, int32_t* tiles, int max_tiles, int tile_rows,
+                              hipStream_t stream) {
     if (tokens <= 0) return 0;
     if (experts <= 0 || experts > MAX_EXPERTS || top <= 0 || top > MAX_TOP || top > experts || stride < experts || parts <= 0) return -1;
     const int pairs = tokens * top;
-    if (max_tiles < (pairs + TILE_ROWS - 1) / TILE_ROWS + (experts < pairs ? experts : pairs)) return -1;
+    if (tile_rows != TILE_ROWS && tile_rows != MFMA_ROWS) return -1;
+    if (max_tiles < (pairs + tile_rows - 1) / tile_rows + (experts < pairs ? experts : pairs)) return -1;
     hipLaunchKernelGGL(moe_route_kernel, dim3((tokens + ROUTE_WAVES - 1) / ROUTE_WAVES), dim3(ROUTE_WAVES * KIPP_WAVE), 0, stream, z, parts,
                        (size_t)tokens * stride, stride, chosen, weight, tokens, experts, top, eps);
     hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, stream, (const int32_t*)chosen, pairs, experts, top, pair_token,
-                       place_of_pair, tiles, max_tiles);
+                       place_of_pair, tiles, max_tiles, tile_rows);
     return KIPP_LAUNCH_CHECK();
 }
 
+// `tile_rows`: the rows of the tiles that `kipp_moe_route` was asked for: 64 takes the matrix cores (bfloat16 x and w, K a multiple of 32), 16 the plain kernel.
 extern "C" int kipp_moe_expert(const void* x, int x_dtype, const int32_t* gather, const void* w, int w_dtype, const int32_t* tiles,
-                               int max_tiles, void* out, int out_dtype, int n_out, int k, int act, hipStream_t stream) {
+                               int max_tiles, void* out, int out_dtype, int n_out, int k, int act, int tile_rows, hipStream_t stream) {
     if (max_tiles <= 0) return 0;
     if (n_out <= 0 || k <= 0 || act < ACT_NONE || act > ACT_GELU_TANH) return -1;
+    if (tile_rows == MFMA_ROWS) {
+        if (x_dtype != KIPP_BF16 || w_dtype != KIPP_BF16 || k % 32) return -2;
+        dim3 grid(max_tiles, (n_out + MFMA_COLS - 1) / MFMA_COLS), block(MFMA_THREADS);
+        if (out_dtype == KIPP_BF16)
+            hipLaunchKernelGGL((moe_expert_mfma_kernel<bf16_t>), grid, block, 0, stream, (const bf16_t*)x, gather, (const bf16_t*)w, tiles,
+                               (bf16_t*)out, n_out, k, act);
+        else if (out_dtype == KIPP_F32)
+            hipLaunchKernelGGL((moe_expert_mfma_kernel<float>), grid, block, 0, stream, (const bf16_t*)x, gather, (const bf16_t*)w, tiles,
+                               (float*)out, n_out, k, act);
+        else
+            return -2;
+        return KIPP_LAUNCH_CHECK();
+    }
+    if (tile_rows != TILE_ROWS) return -1;
     dim3 grid(max_tiles, (n_out + EXPERT_COLS - 1) / EXPERT_COLS), block(EXPERT_COLS);
 #define KIPP_ME(TX, TW, TO)                                                                                                  \
     hipLaunchKernelGGL((moe_expert_kernel<TX, TW, TO>), grid, block, 0, stream, (const TX*)x, gather, (const TW*)w, tiles, \

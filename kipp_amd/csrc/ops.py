@@ -717,38 +717,45 @@ def scan_finish(o_raw: torch.Tensor, gates: torch.Tensor, gate_at: int, norm_w: 
 
 ACTIVATIONS = {"silu": 0, "relu": 1, "gelu": 2, "gelu_tanh": 3}
 MOE_TILE_ROWS = 16
+MOE_MFMA_ROWS = 64     # rows of a tile of the experts' products on the matrix cores
 
 
-def moe_max_tiles(tokens: int, experts: int, top: int) -> int:
-    """Tiles of up to 16 rows that the sorted pairs of a step can need at most (every expert may end in a partial one)."""
+def moe_tile_rows(dtype: torch.dtype, *contractions: int) -> int:
+    """Rows of the tiles that the experts' products take: 64 on the matrix cores (bfloat16, every contraction a multiple of
+    32), else 16."""
+    return MOE_MFMA_ROWS if dtype == torch.bfloat16 and all(k % 32 == 0 for k in contractions) else MOE_TILE_ROWS
+
+
+def moe_max_tiles(tokens: int, experts: int, top: int, tile_rows: int = 16) -> int:
+    """Tiles of up to `tile_rows` rows that the sorted pairs of a step can need at most (every expert may end in a partial one)."""
     pairs = tokens * top
-    return -(-pairs // MOE_TILE_ROWS) + min(experts, pairs)
+    return -(-pairs // tile_rows) + min(experts, pairs)
 
 
 def moe_route(z: torch.Tensor, experts: int, top: int, eps: float, chosen: torch.Tensor, weight: torch.Tensor,
-              pair_token: torch.Tensor, place_of_pair: torch.Tensor, tiles: torch.Tensor):
+              pair_token: torch.Tensor, place_of_pair: torch.Tensor, tiles: torch.Tensor, tile_rows: int = 16):
     """From router logits `z` (float32 [tokens, >= experts] or slabs): softmax over the experts, the `top` largest a token
     (`chosen`, int32 [tokens, top]) with weights p / (sum of the chosen p + eps) (`weight`, float32 [tokens, top]); then the
     pairs sorted by expert: `pair_token` [pairs] the token of every sorted row, `place_of_pair` [pairs] the row of pair
-    (token, choice), `tiles` int32 [max_tiles, 3] = (expert, first row, rows), unused tiles with 0 rows."""
+    (token, choice), `tiles` int32 [max_tiles, 3] = (expert, first row, rows) of up to `tile_rows` rows, unused tiles with 0 rows."""
     _dev(z, chosen, weight, pair_token, place_of_pair, tiles)
     parts, n, stride = _slabs(z, "moe_route")
     for t, name in ((chosen, "chosen"), (pair_token, "pair_token"), (place_of_pair, "place_of_pair"), (tiles, "tiles")):
         _i32(t, name)
     _need(0 < top <= experts <= 1024 and top <= 32 and stride >= experts, "moe_route: up to 1,024 experts, up to 32 a token")
     _need(chosen.shape == (n, top) and weight.shape == (n, top) and weight.dtype == torch.float32 and pair_token.numel() == n * top
-          and place_of_pair.numel() == n * top and tiles.dim() == 2 and tiles.shape[1] == 3 and tiles.shape[0] >= moe_max_tiles(n, experts, top),
+          and place_of_pair.numel() == n * top and tiles.dim() == 2 and tiles.shape[1] == 3 and tiles.shape[0] >= moe_max_tiles(n, experts, top, tile_rows),
           "moe_route: output shapes")
-    fn = _fn("moe", "kipp_moe_route", [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr])
+    fn = _fn("moe", "kipp_moe_route", [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(z), parts, stride, _ptr(chosen), _ptr(weight), n, experts, top, float(eps), _ptr(pair_token), _ptr(place_of_pair), _ptr(tiles),
-              tiles.shape[0], _stream()), "moe_route")
+              tiles.shape[0], int(tile_rows), _stream()), "moe_route")
     return chosen, weight
 
 
 def moe_expert(x: torch.Tensor, gather: Optional[torch.Tensor], w: torch.Tensor, tiles: torch.Tensor, out: torch.Tensor,
-               activation: Optional[str] = None) -> torch.Tensor:
+               activation: Optional[str] = None, tile_rows: int = 16) -> torch.Tensor:
     """Every tile's rows against its expert's matrix: out[row] = act(w[expert] x_row), x_row = x[gather[row]] (or x[row]);
-    `w` [experts, n_out, k], `out` [sorted rows, n_out]."""
+    `w` [experts, n_out, k], `out` [sorted rows, n_out].  `tile_rows`: what `moe_route` was given (64: the matrix cores)."""
     _dev(x, gather, w, tiles, out)
     _i32(tiles, "tiles")
     if gather is not None:
@@ -757,9 +764,11 @@ def moe_expert(x: torch.Tensor, gather: Optional[torch.Tensor], w: torch.Tensor,
           "moe_expert: x [rows, k], w [experts, n_out, k] of one type, out [rows, n_out]")
     _need(out.shape[0] == (gather.numel() if gather is not None else x.shape[0]), "moe_expert: one output row a sorted row")
     _need(activation is None or activation in ACTIVATIONS, f"moe_expert: activation is one of {sorted(ACTIVATIONS)}")
-    fn = _fn("moe", "kipp_moe_expert", [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _need(tile_rows == MOE_TILE_ROWS or (tile_rows == MOE_MFMA_ROWS and x.dtype == torch.bfloat16 and w.shape[2] % 32 == 0),
+          "moe_expert: tiles of 16 rows, or of 64 for bfloat16 with K a multiple of 32")
+    fn = _fn("moe", "kipp_moe_expert", [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(x), _code(x), _ptr(gather), _ptr(w), _code(w), _ptr(tiles), tiles.shape[0], _ptr(out), _code(out), w.shape[1], w.shape[2],
-              -1 if activation is None else ACTIVATIONS[activation], _stream()), "moe_expert")
+              -1 if activation is None else ACTIVATIONS[activation], int(tile_rows), _stream()), "moe_expert")
     return out
 
 
@@ -976,8 +985,10 @@ def compute_units(device=None) -> int:
 def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                      rows: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
                      n_q: int, n_kv: int, head_dim: int, scale: float, window: int, max_context: int,
-                     workspace: tuple, grid_splits: Optional[int] = None) -> torch.Tensor:
+                     workspace: tuple, grid_splits: Optional[int] = None, capped: bool = False) -> torch.Tensor:
     """Attention of single query tokens (batch rows `rows`) over their pages.
+    `capped`: the build whose scores pass tanh: `scale` is then the cap c, and q comes multiplied by (the score's
+    scale / c), so that a weight is exp(c tanh(q . k scale / c) - maximum).
     `max_context`: the longest context among them (sizes the grid); `workspace`:
     (part_acc, part_ml, arrivals) from `attention_decode_workspace` (without `arrivals`, or with None for it,
     the splits are merged by a launch of its own instead of by the last workgroup of every head)."""
@@ -997,6 +1008,8 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
           and part_acc.numel() >= n_items * n_q * max_splits * head_dim and need <= max_splits,
           "attention_decode: workspace too small for this context")
     defines = {"HEAD_DIM": head_dim, "GROUP": group}
+    if capped:
+        defines["SOFTCAP"] = 1
     fn = _fn("attention_decode", "kipp_attention_decode",
              [_c_ptr] * 10 + [_c_int] * 6 + [_c_float, _c_int, _c_int, _c_int, _c_ptr, _c_ptr], defines)
     _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(part_acc), _ptr(part_ml), _ptr(rows),
@@ -1107,9 +1120,11 @@ def attention_decode_workspace(n_items: int, n_q: int, head_dim: int, max_contex
 def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                       item_seq: torch.Tensor, item_tile: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
                       positions: torch.Tensor, block_table: torch.Tensor, n_q: int, n_kv: int, head_dim: int,
-                      scale: float, window: int = 0, tile_rows: int = 128, cuts=None) -> torch.Tensor:
+                      scale: float, window: int = 0, tile_rows: int = 128, cuts=None, capped: bool = False) -> torch.Tensor:
     """Attention of prompt portions: work item i is the `item_tile[i]`-th tile
     of `tile_rows` (128, 64 or 32) query rows of sequence `item_seq[i]`.
+    `capped`: the build whose scores pass tanh: `scale` is then the cap c, and q comes multiplied by (the score's
+    scale / c), so that a weight is exp(c tanh(q . k scale / c) - maximum).
 
     `cuts` = (split_keys, item_split, merge_rows, merge_cuts, workspace): the keys are cut at multiples of
     `split_keys` (a multiple of 64), work item i takes cut `item_split[i]` of its tile's keys, and the rows
@@ -1138,7 +1153,7 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
               "attention_prefill: cuts need no window, a multiple of 64 keys, one cut per work item and a workspace for every row")
     fn = _fn("attention_prefill", "kipp_attention_prefill",
              [_c_ptr] * 10 + [_c_int] * 6 + [_c_float, _c_int, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int,
-                                             _c_ptr], {"HEAD_DIM": head_dim})
+                                             _c_ptr], {"HEAD_DIM": head_dim, "SOFTCAP": 1} if capped else {"HEAD_DIM": head_dim})
     _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(item_seq), _ptr(item_tile), _ptr(q_start),
               _ptr(q_len), _ptr(positions), _ptr(block_table), block_table.shape[1], item_seq.numel(), n_q, n_kv,
               head_dim, k_cache.shape[2], float(scale), int(window), int(tile_rows), _ptr(item_split), int(split_keys),

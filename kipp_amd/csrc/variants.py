@@ -65,6 +65,7 @@ def prebuilt() -> List[Spec]:
 ATTENTION = [(128, 16), (128, 1), (16, 3), (48, 3), (64, 1), (32, 16), (256, 4), (80, 3), (256, 2), (16, 1), (32, 2), (16, 6), (64, 4), (256, 16)]   # (head size, group)
 EARLY_STREAM = [(128, 4), (48, 3), (16, 2)]      # the kernel for long contexts takes over at 1,024 keys
 WHOLE_CONTEXTS = [(128, 4), (128, 16)]           # the whole-context kernel at few sequences
+CAPPED = [(32, 2), (128, 4), (64, 1), (16, 2), (32, 1)]      # scores capped by tanh: (head size, group)
 MIXED_HEADS = [(6, 3, 32, 16), (4, 4, 32, 32), (8, 2, 64, 48), (12, 4, 32, 64), (2, 1, 96, 16), (32, 8, 32, 16), (4, 2, 32, 16), (32, 8, 128, 128), (16, 4, 32, 16)]   # (heads, key/value heads, key size, value size) of the attention with mixed heads
 
 
@@ -78,6 +79,11 @@ def check_builds() -> List[Spec]:
         out.append(("attention_decode", {"HEAD_DIM": head_dim, "GROUP": group, "STREAM_FROM": 1024}))
     for head_dim, group in WHOLE_CONTEXTS:
         out.append(("attention_decode", {"HEAD_DIM": head_dim, "GROUP": group, "RING_FROM_PAIRS": 1}))
+    for head_dim, group in CAPPED:
+        out.append(("attention_prefill", {"HEAD_DIM": head_dim, "SOFTCAP": 1}))
+        out.append(("attention_decode", {"HEAD_DIM": head_dim, "GROUP": group, "SOFTCAP": 1}))
+    out.append(("attention_decode", {"HEAD_DIM": 128, "GROUP": 4, "SOFTCAP": 1, "STREAM_FROM": 1024}))
+    out.append(("attention_decode", {"HEAD_DIM": 128, "GROUP": 4, "SOFTCAP": 1, "RING_FROM_PAIRS": 1}))
     from .ops import mixed_attention_builds
     for heads, kv_heads, head_dim, v_dim in MIXED_HEADS:
         out += [("attention_mixed_mfma", defines) for defines in mixed_attention_builds(heads, kv_heads, head_dim, v_dim)]

@@ -138,12 +138,14 @@ class RoutedMLP:
         weight = rt.empty((n, s.top), torch.float32)
         pair_token = torch.empty((pairs,), dtype=torch.int32, device=dev)
         place = torch.empty((pairs,), dtype=torch.int32, device=dev)
-        tiles = torch.empty((ops.moe_max_tiles(n, s.experts, s.top), 3), dtype=torch.int32, device=dev)
-        ops.moe_route(z, s.experts, s.top, s.weight_eps, chosen, weight, pair_token, place, tiles)
+        # bfloat16 experts whose two contractions are multiples of 32 run on the matrix cores, in tiles of 64 rows
+        tile_rows = ops.moe_tile_rows(self.w_up.dtype, s.hidden_size, s.expert_size)
+        tiles = torch.empty((ops.moe_max_tiles(n, s.experts, s.top, tile_rows), 3), dtype=torch.int32, device=dev)
+        ops.moe_route(z, s.experts, s.top, s.weight_eps, chosen, weight, pair_token, place, tiles, tile_rows=tile_rows)
         if x.dtype != self.w_up.dtype:
             x = ops.cast(x, rt.empty(x.shape, self.w_up.dtype))
-        inner = ops.moe_expert(x, pair_token, self.w_up, tiles, rt.empty((pairs, s.expert_size), self.w_up.dtype), s.activation)
-        y = ops.moe_expert(inner, None, self.w_down, tiles, rt.empty((pairs, s.hidden_size), torch.float32))
+        inner = ops.moe_expert(x, pair_token, self.w_up, tiles, rt.empty((pairs, s.expert_size), self.w_up.dtype), s.activation, tile_rows=tile_rows)
+        y = ops.moe_expert(inner, None, self.w_down, tiles, rt.empty((pairs, s.hidden_size), torch.float32), tile_rows=tile_rows)
         shared = None
         if s.shared_size is not None:
             mid = ops.activate(rt.linear(x, self.w_shared_up, slabs=True), rt.empty((n, s.shared_size), rt.act_dtype), s.activation)

@@ -70,12 +70,13 @@ class Attention:
         that share a key/value head).  Under float32, and for more than 16 heads a group, the generic
         attention kernel runs, which every model has."""
         out = [("rope_kv", None) if spec.plain else ("head_prepare", None), ("attention_generic", None)]
-        if dtype != "bfloat16" or spec.head_dim % 16 or spec.value_dim != spec.head_dim or spec.softcap is not None:
+        if dtype != "bfloat16" or spec.head_dim % 16 or spec.value_dim != spec.head_dim:
             return out
         group = spec.num_heads // spec.num_kv_heads
-        out.append(("attention_prefill", {"HEAD_DIM": spec.head_dim}))
+        capped = {"SOFTCAP": 1} if spec.softcap is not None else {}      # capped scores: builds of their own
+        out.append(("attention_prefill", {"HEAD_DIM": spec.head_dim, **capped}))
         if group <= 16:
-            out.append(("attention_decode", {"HEAD_DIM": spec.head_dim, "GROUP": group}))
+            out.append(("attention_decode", {"HEAD_DIM": spec.head_dim, "GROUP": group, **capped}))
         return out
 
     def load(self, tensors):
@@ -92,6 +93,11 @@ class Attention:
             self.q_norm = tensors[names[4]]
             self.k_norm = tensors[names[5]]
         self.head_temp = tensors[s.head_temp] if s.head_temp is not None else None
+        self.head_temp_capped = None
+        if s.softcap is not None:
+            # for the matrix-core kernels, which cap what they are given: queries times (scale / cap) beside the head's factor
+            ones = torch.ones(s.num_heads, dtype=torch.float32, device=self.w_o.rows.device)
+            self.head_temp_capped = ((self.head_temp.float() if self.head_temp is not None else ones) * (self.scale / s.softcap)).contiguous()
         self.bias = None
         if s.bias:
             held = [tensors[name] for name in (s.bias_names if s.own_kv else s.bias_names[:1])]
@@ -178,12 +184,14 @@ class Attention:
         norm = "none" if s.qk_norm_eps is None else ("weighted" if s.qk_norm_weight else "plain")
         coef, every = s.q_temp if s.q_temp is not None else (0.0, 0)
         # (without projections of its own only q was projected: its columns stand at the row's start all the same)
+        fast = rt.dtype == "bfloat16" and d % 16 == 0 and d == dv \
+            and rt.ops.attention_fast_ok(s.num_heads, s.num_kv_heads, cache.page_size, table.shape[1])
+        capped = fast and s.softcap is not None
         q = rt.ops.head_prepare(proj, rt.empty((n, s.q_dim), rt.act_dtype), cache.k, cache.v, batch.positions,
                                 batch.seq_of_token, table, s.num_heads, s.num_kv_heads, d, dv, self.bias, norm,
                                 s.qk_norm_eps or 0.0, self.q_norm, self.k_norm, coef, every,
-                                write_kv=cache.writable and s.own_kv, q_head_scale=self.head_temp, v_norm_eps=s.v_norm_eps)
-        fast = rt.dtype == "bfloat16" and d % 16 == 0 and d == dv and s.softcap is None \
-            and rt.ops.attention_fast_ok(s.num_heads, s.num_kv_heads, cache.page_size, table.shape[1])
+                                write_kv=cache.writable and s.own_kv,
+                                q_head_scale=self.head_temp_capped if capped else self.head_temp, v_norm_eps=s.v_norm_eps)
         if rt.dtype == "bfloat16" and not fast:
             rt.generic_attention_launches += 1
         out = rt.empty((n, s.out_dim), rt.act_dtype)
@@ -197,17 +205,19 @@ def paged_attention(rt, batch, q, out, k_cache, v_cache, page_size, table, n_q, 
     [tokens, n_q dv].  `fast`: the matrix-core kernels (prompt portions and single tokens each by their own; they
     need d == dv, or `v_cache` being `k_cache`, a value then being as wide as its key's row); else the generic kernel,
     which takes values of their own width (`v_cache` may be `k_cache` there too: a value is the first dv numbers
-    of its key's row).  `softcap` c > 0: a scaled score s becomes c tanh(s / c) (the generic kernel).  `owner`: a mixer whose `_prefill_work(batch)` and `_workspace(batch)` make the work list and the
+    of its key's row).  `softcap` c > 0: a scaled score s becomes c tanh(s / c) (with `fast`, q must come multiplied by scale / c).  `owner`: a mixer whose `_prefill_work(batch)` and `_workspace(batch)` make the work list and the
     decode workspace (else they are made here for these sizes)."""
     if fast:
+        # capped scores: the builds that pass what they are given through tanh; q then comes times (scale / cap), and the cap is the scale
+        capped = bool(softcap)
         if batch.n_portions:
             item_seq, item_tile, cuts = owner._prefill_work(batch) if owner is not None else prefill_work(rt, batch, n_q, d, window)
             rt.ops.attention_prefill(q, k_cache, v_cache, out, item_seq, item_tile, batch.q_start, batch.q_len, batch.positions,
-                                     table, n_q, n_kv, d, scale, window or 0, cuts=cuts)
+                                     table, n_q, n_kv, d, softcap if capped else scale, window or 0, cuts=cuts, capped=capped)
         if batch.n_decode:
             rt.ops.attention_decode(q, k_cache, v_cache, out, batch.decode_rows, batch.positions, batch.seq_of_token, table,
-                                    n_q, n_kv, d, scale, window or 0, batch.max_decode_ctx,
-                                    owner._workspace(batch) if owner is not None else decode_workspace(rt, batch, n_q, d))
+                                    n_q, n_kv, d, softcap if capped else scale, window or 0, batch.max_decode_ctx,
+                                    owner._workspace(batch) if owner is not None else decode_workspace(rt, batch, n_q, d), capped=capped)
     elif d == dv and v_cache is not k_cache and d <= 256 and not softcap:
         # the float32 path, and geometries the matrix-core kernels refuse (groups above 16, odd page sizes)
         rt.ops.paged_attention_generic(q, k_cache, v_cache, out, batch.positions, batch.seq_of_token, table, n_q, n_kv, d,

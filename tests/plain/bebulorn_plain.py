@@ -185,9 +185,16 @@ def expert(h, w, p):
     return linear(gelu_erf(linear(h, w[p + "up"])), w[p + "down"])
 
 
+ROUTE_MARGINS = None     # a list, when someone wants them: every call of `route` appends its tokens' margins [T]
+
+
 def route(h, w_router, top):
-    """(chosen experts [T, top], their weights [T, top])."""
+    """(chosen experts [T, top], their weights [T, top]).  A token's margin is the gap between the logit of its last
+    chosen expert and the largest one left out: where it is small, reduced precision may choose otherwise."""
     z = linear(h, w_router)
+    if ROUTE_MARGINS is not None:
+        ordered = -np.sort(-z, axis=1)
+        ROUTE_MARGINS.append(ordered[:, top - 1] - ordered[:, top] if top < z.shape[1] else np.full(z.shape[0], np.inf))
     e = np.exp(z - z.max(axis=1, keepdims=True))
     s = e / e.sum(axis=1, keepdims=True)
     chosen = np.argsort(-s, axis=1, kind="stable")[:, :top]

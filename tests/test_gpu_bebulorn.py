@@ -54,28 +54,43 @@ def folders(tmp_path_factory):
 
 
 _plain_cache = {}
+_margin_cache = {}
 
 
 def plain_logits(folder, tokens):
     key = (folder, tuple(tokens))
     if key not in _plain_cache:
         cfg, w = P.load_folder(folder)
-        _plain_cache[key] = P.forward_whole(cfg, w, list(tokens))
+        P.ROUTE_MARGINS = []
+        try:
+            _plain_cache[key] = P.forward_whole(cfg, w, list(tokens))
+            _margin_cache[id(_plain_cache[key])] = np.min(P.ROUTE_MARGINS, axis=0) if P.ROUTE_MARGINS else None
+        finally:
+            P.ROUTE_MARGINS = None
     return _plain_cache[key]
 
 
 FLIPS = 0.5       # share of a request's positions that may lie beyond the bfloat16 bound (see `close`)
+CLOSE_CALL = 0.3  # a router's margin (in logits) below which bfloat16 rows may choose another expert
 
 
 def close(got, ref, tol, what):
-    """Every position's normalised squared error within `tol`.  Under the bfloat16 bound a share of the positions may lie
-    beyond it: a router's choice between two experts whose scores differ by less than the rounding of the rows it reads
-    falls either way, and the position (and, through memories that forget slowly or never, every one after it) then
-    differs by much more than rounding.  The float32 runs of the same cases allow no such position; what is wrong for most positions (a window, a
-    state, a page) fails either bound."""
+    """Every position's normalised squared error within `tol`.  Under the bfloat16 bound a router's choice between two
+    experts whose logits differ by less than the rounding of the rows it reads falls either way, and the position (and,
+    through memories that forget slowly or never, every one after it) then differs by much more than rounding: a request
+    passes if every position beyond the bound stands at or behind a close call of the plain implementation's routers
+    (`ref` from `plain_logits`, which keeps their margins), or if no more than a share of its positions lie beyond it.
+    The float32 runs of the same cases allow no such position; what is wrong for most positions (a window, a state, a
+    page) fails either bound."""
     assert got.shape == ref.shape and np.isfinite(got).all(), what
-    errs = sorted(float(np.sum((g - r) ** 2) / np.sum(r ** 2)) for g, r in zip(got.astype(np.float64), ref))
+    each = [float(np.sum((g - r) ** 2) / np.sum(r ** 2)) for g, r in zip(got.astype(np.float64), ref)]
+    errs = sorted(each)
     spared = int(FLIPS * len(errs)) if tol >= TOL["bfloat16"] else 0
+    margins = _margin_cache.get(id(ref)) if spared else None
+    if margins is not None and len(margins) == len(each):
+        called = np.minimum.accumulate(margins) < CLOSE_CALL          # a close call at or before the position
+        if all(e <= tol or c for e, c in zip(each, called)):
+            return
     worst = errs[len(errs) - 1 - spared]
     over = sum(e > tol for e in errs)
     assert worst <= tol, f"{what}: NMSE {worst:.3e} exceeds {tol:.1e} ({over} of {len(errs)} positions beyond it, {spared} spared)"
@@ -251,7 +266,8 @@ def test_scan_finish(gate, span, w_len):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("experts, top, tokens, width, inner", [(16, 2, 37, 64, 96), (5, 3, 1, 72, 40), (8, 1, 300, 40, 24), (70, 4, 129, 32, 520), (3, 3, 20, 300, 16)])
+@pytest.mark.parametrize("experts, top, tokens, width, inner", [(16, 2, 37, 64, 96), (5, 3, 1, 72, 40), (8, 1, 300, 40, 24), (70, 4, 129, 32, 520), (3, 3, 20, 300, 16),
+                                                                (4, 2, 333, 320, 96), (6, 1, 70, 32, 32), (40, 4, 5, 288, 160)])
 def test_routed_feed_forward_kernels(dtype, experts, top, tokens, width, inner):
     """Choice and weights (with logits that tie), the sort into runs of one expert (some experts get nothing, some more than
     a tile), both expert products and the weighted sum with a shared part in slabs: against loops over tokens."""
@@ -270,8 +286,10 @@ def test_routed_feed_forward_kernels(dtype, experts, top, tokens, width, inner):
     pairs = tokens * top
     chosen, weight = torch.empty((tokens, top), dtype=torch.int32, device="cuda:0"), torch.empty((tokens, top), device="cuda:0")
     pair_token, place = torch.empty(pairs, dtype=torch.int32, device="cuda:0"), torch.empty(pairs, dtype=torch.int32, device="cuda:0")
-    tiles = torch.full((ops.moe_max_tiles(tokens, experts, top), 3), -7, dtype=torch.int32, device="cuda:0")
-    ops.moe_route(f32(z), experts, top, 1e-20, chosen, weight, pair_token, place, tiles)
+    tile_rows = ops.moe_tile_rows(ty, width, inner)       # 64 (the matrix cores) for bfloat16 where both contractions are multiples of 32
+    assert tile_rows == (64 if dtype == "bfloat16" and width % 32 == 0 and inner % 32 == 0 else 16)
+    tiles = torch.full((ops.moe_max_tiles(tokens, experts, top, tile_rows), 3), -7, dtype=torch.int32, device="cuda:0")
+    ops.moe_route(f32(z), experts, top, 1e-20, chosen, weight, pair_token, place, tiles, tile_rows=tile_rows)
     zz = z.astype(np.float64).sum(axis=0)[:, :experts]
     e = np.exp(zz - zz.max(axis=1, keepdims=True))
     s = e / e.sum(axis=1, keepdims=True)
@@ -292,13 +310,13 @@ def test_routed_feed_forward_kernels(dtype, experts, top, tokens, width, inner):
     assert np.all(np.diff(expert_of_row) >= 0)
     covered = np.zeros(pairs, dtype=int)
     for ex, first, rows in tl:
-        assert 0 <= rows <= 16
+        assert 0 <= rows <= tile_rows
         if rows:
             assert np.all(expert_of_row[first:first + rows] == ex)
             covered[first:first + rows] += 1
     assert np.all(covered == 1)
-    mid = ops.moe_expert(dev(x, ty), pair_token, dev(w_up, ty), tiles, torch.empty((pairs, inner), dtype=ty, device="cuda:0"), "gelu")
-    y = ops.moe_expert(mid, None, dev(w_down, ty), tiles, torch.empty((pairs, width), device="cuda:0"))
+    mid = ops.moe_expert(dev(x, ty), pair_token, dev(w_up, ty), tiles, torch.empty((pairs, inner), dtype=ty, device="cuda:0"), "gelu", tile_rows=tile_rows)
+    y = ops.moe_expert(mid, None, dev(w_down, ty), tiles, torch.empty((pairs, width), device="cuda:0"), tile_rows=tile_rows)
     out = ops.moe_combine(y, place, weight, f32(shared), torch.empty((tokens, width), device="cuda:0")).cpu().numpy()
     ref = shared.astype(np.float64).sum(axis=0)
     wt = weight.cpu().numpy().astype(np.float64)
@@ -373,6 +391,82 @@ def test_capped_attention_with_a_key_that_stands_out(dtype, H_, G, d, dv, window
                 assert np.allclose(got[:, 0], np.sqrt(dv), rtol=2e-2), (key, list(rows)[:2], got[:, 0])
             else:
                 assert np.all(np.abs(got[:, 0]) < 0.9 * np.sqrt(dv)), (key, list(rows)[:2], got[:, 0])
+
+
+@pytest.mark.parametrize("n_q, n_kv, d, page, window, build", [
+    (4, 2, 32, 16, 40, None), (8, 2, 128, 16, 100, None), (3, 3, 64, 8, 0, None), (8, 2, 128, 16, 0, None),
+    (8, 2, 128, 16, 0, "STREAM_FROM"), (8, 2, 128, 16, 1500, "STREAM_FROM"), (8, 2, 128, 16, 300, "RING_FROM_PAIRS"), (8, 2, 128, 16, 0, "RING_FROM_PAIRS")])
+def test_capped_attention_on_the_matrix_cores(n_q, n_kv, d, page, window, build):
+    """The builds of the matrix-core attention that pass a score through tanh and take the cap as their scale, for prompt
+    portions and for single tokens (also the kernels for long contexts and for whole contexts, built so that small inputs
+    reach them), against softmax(cap tanh(q . k)) v written out here, with scores on both sides of the cap's bend."""
+    import torch
+    from kipp_amd.csrc import ops
+    rng = np.random.default_rng(n_q + d + window + len(build or ""))
+    cap = 12.0
+    seq_lens = [1, 70, 300, 257, 129] + ([2300, 1025] if build else [])
+    q_lens = [1, 70, 130, 2, 129] + ([200, 1] if build else [])
+    blocks = [-(-n // page) for n in seq_lens]
+    perm = rng.permutation(sum(blocks) + 3)
+    table = np.zeros((len(seq_lens), max(blocks)), dtype=np.int32)
+    at = 0
+    for i, b in enumerate(blocks):
+        table[i, :b] = perm[at:at + b]
+        at += b
+    k = torch.tensor(rng.normal(size=(len(perm), n_kv, page, d)), dtype=torch.bfloat16)
+    v = torch.tensor(rng.normal(size=(len(perm), n_kv, page, d)) + 1.0, dtype=torch.bfloat16)
+
+    def keys_of(cache, seq, n):
+        return np.stack([cache[table[seq, j // page], :, j % page, :].double().numpy() for j in range(n)])      # [n, n_kv, d]
+
+    def expected(qrow, seq, pos):
+        ks, vs = keys_of(k, seq, pos + 1), keys_of(v, seq, pos + 1)
+        lo = max(0, pos - window + 1) if window else 0
+        out = np.zeros((n_q, d))
+        for h in range(n_q):
+            g = h // (n_q // n_kv)
+            sc = cap * np.tanh(ks[lo:, g] @ qrow[h])
+            w = np.exp(sc - sc.max())
+            out[h] = (w / w.sum()) @ vs[lo:, g]
+        return out
+
+    inner = ops._fn
+    if build:
+        ops._fn = lambda lib, name, argtypes, defines=None: inner(lib, name, argtypes, dict(defines, **{build: 1024 if build == "STREAM_FROM" else 1}) if lib == "attention_decode" else defines)
+    try:
+        # prompt portions: the last q_len tokens of every sequence
+        positions, seq_of, q_start = [], [], []
+        for i, (n, ql) in enumerate(zip(seq_lens, q_lens)):
+            q_start.append(len(positions))
+            positions += list(range(n - ql, n))
+            seq_of += [i] * ql
+        t = len(positions)
+        q = torch.tensor(rng.normal(size=(t, n_q * d)) * (1.6 / np.sqrt(d)), dtype=torch.bfloat16)       # as the mixer hands them over: times scale / cap
+        items = [(i, tile) for i, ql in enumerate(q_lens) for tile in range(-(-ql // 128))]
+        out = ops.attention_prefill(q.cuda(), k.cuda(), v.cuda(), torch.zeros(t, n_q * d, dtype=torch.bfloat16, device="cuda:0"),
+                                    i32([i for i, _ in items]), i32([tile for _, tile in items]), i32(q_start), i32(q_lens), i32(positions),
+                                    i32(table), n_q, n_kv, d, cap, window, capped=True).float().cpu().numpy().reshape(t, n_q, d)
+        qd = q.double().numpy().reshape(t, n_q, d)
+        for row in sorted(set(list(range(0, t, 17)) + q_start + [s + ql - 1 for s, ql in zip(q_start, q_lens)])):
+            ref = expected(qd[row], seq_of[row], positions[row])
+            assert np.abs(out[row] - ref).max() < 2e-2 * max(1.0, np.abs(ref).max()), ("portion", row, seq_of[row], positions[row])
+        # single tokens: the last token of every sequence, rows that are not the first of their batch
+        n_seq = len(seq_lens)
+        rows = list(range(2, n_seq + 2))
+        pos1, seq1 = [0, 0] + [n - 1 for n in seq_lens], [0, 0] + list(range(n_seq))
+        q1 = torch.tensor(rng.normal(size=(n_seq + 2, n_q * d)) * (1.6 / np.sqrt(d)), dtype=torch.bfloat16)
+        out1 = torch.zeros(n_seq + 2, n_q * d, dtype=torch.bfloat16, device="cuda:0")
+        ws = ops.attention_decode_workspace(n_seq, n_q, d, max(seq_lens), "cuda:0")
+        ops.attention_decode(q1.cuda(), k.cuda(), v.cuda(), out1, i32(rows), i32(pos1), i32(seq1), i32(table), n_q, n_kv, d, cap, window,
+                             max(seq_lens), ws, capped=True)
+        got = out1.float().cpu().numpy().reshape(n_seq + 2, n_q, d)
+        q1d = q1.double().numpy().reshape(n_seq + 2, n_q, d)
+        for r in rows:
+            ref = expected(q1d[r], seq1[r], pos1[r])
+            assert np.abs(got[r] - ref).max() < 2e-2 * max(1.0, np.abs(ref).max()), ("single token", r, pos1[r])
+        assert not got[:2].any()
+    finally:
+        ops._fn = inner
 
 
 # =============================================================================== the engine
