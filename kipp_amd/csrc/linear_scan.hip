@@ -5,15 +5,16 @@
 //     delta   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q      (q, k, v, beta, g made ready by `prepare`)
 //
 // `scan`: a workgroup takes (entry, head, a run of columns of S) and walks the entry's tokens in order.  A column of S is
-// shared by L lanes side by side in a wave (L a power of two, 8 or 16 rows a lane, row r with lane r % L), so the sums over
-// rows end in moves between the lanes of a wave and the walk has no barrier of its own; tokens come in chunks through
-// LDS.  What is computed for a token depends on the state and the token alone, never on where a chunk or a portion
+// shared by L lanes side by side in a wave (L a power of two, 8 or 16 rows in a run a lane), so the sums over rows end in
+// data-parallel moves between the lanes of a wave and the walk has no barrier of its own; tokens come in chunks through
+// LDS, four at a time, so that the sums of four tokens' outputs run side by side.  What is computed for a token depends on the state and the token alone, never on where a chunk or a portion
 // begins: prompt portions and single tokens give the same bits.  State in the slot: S as [head][column][row].
 //
 // `prepare` (delta rule): the short causal convolutions over q | k | v with their silu, the unit norm of every q and k head,
 // beta and g, from the input product and the slot's last taps - 1 inputs; `conv_keep` then writes the slot's new last
 // inputs.  `finish`: a root mean square over a span of columns, a weight, a gate.
 #include "common.h"
+#include "lane_sums.h"
 #include <math.h>
 
 #define SCAN_THREADS 256
@@ -23,60 +24,109 @@ __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z));
 __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
 __device__ __forceinline__ float softplus_f(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
 
-// sum over the L lanes that share a column (they are neighbours in the wave); every one of them gets the same bits
-__device__ __forceinline__ float column_sum(float v, int lanes) {
-    for (int off = 1; off < lanes; off <<= 1) v += __shfl_xor(v, off, KIPP_WAVE);
-    return v;
+// One token of the walk for a lane's R rows of a column: the new rows, and the lane's share of o (summed over the
+// column's lanes by the caller, so that the sums of several tokens run side by side).  The same code whether the token
+// stands alone or among others: a position's bits do not depend on how the tokens were cut.
+template <int MODE, int R, int LANES>
+__device__ __forceinline__ float scan_token(float (&S)[R], const float* __restrict__ kt, const float* __restrict__ qt, float vv,
+                                            float decay, float beta, float g) {
+    float k[R], q[R];
+#pragma unroll
+    for (int i = 0; i < R; i += 4) {
+        const float4 k4 = *(const float4*)(kt + i), q4 = *(const float4*)(qt + i);
+        k[i] = k4.x; k[i + 1] = k4.y; k[i + 2] = k4.z; k[i + 3] = k4.w;
+        q[i] = q4.x; q[i + 1] = q4.y; q[i + 2] = q4.z; q[i + 3] = q4.w;
+    }
+    float acc = 0.0f;
+    if (MODE == 0) {
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            S[i] = fmaf(decay, S[i], k[i] * vv);
+            acc = fmaf(S[i], q[i], acc);
+        }
+    } else {
+        float read = 0.0f;
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            S[i] *= g;
+            read = fmaf(S[i], k[i], read);
+        }
+        const float u = beta * (vv - column_sum<LANES>(read));
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            S[i] = fmaf(k[i], u, S[i]);
+            acc = fmaf(S[i], q[i], acc);
+        }
+    }
+    return acc;
 }
 
-// MODE 0: fixed decay, inputs through silu.  MODE 1: delta rule, inputs as they are.
-template <int MODE, int R>
+// MODE 0: fixed decay, inputs through silu.  MODE 1: delta rule, inputs as they are.  A column of S is shared by LANES
+// lanes side by side, lane `sub` with the R rows sub R .. sub R + R - 1 (read from LDS 16 bytes at a time; rows beyond d
+// are zeros there and stay zeros in S).
+template <int MODE, int R, int LANES>
 __global__ void __launch_bounds__(SCAN_THREADS)
 matrix_scan_kernel(const float* __restrict__ src, int stride, int q_at, int k_at, int v_at, int beta_at, int g_at,
                    const float* __restrict__ decays, float* __restrict__ state, size_t state_stride,
                    const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ slots,
-                   float* __restrict__ o_raw, int heads, int qk_rep, int d, int dv, int lanes, int chunk) {
-    extern __shared__ float lds[];
-    const int cols = SCAN_THREADS / lanes;
-    float* k_s = lds;                       // [chunk][d]
-    float* q_s = k_s + (size_t)chunk * d;   // [chunk][d]
-    float* v_s = q_s + (size_t)chunk * d;   // [chunk][cols]
-    float* s_s = v_s + (size_t)chunk * cols;  // [chunk][2]: beta, g
+                   float* __restrict__ o_raw, int heads, int qk_rep, int d, int dv, int chunk) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    constexpr int COLS = SCAN_THREADS / LANES;
+    constexpr int DP = R * LANES;           // a key's numbers in LDS, filled up with zeros
+    float* k_s = lds;                       // [chunk][DP]
+    float* q_s = k_s + (size_t)chunk * DP;  // [chunk][DP]
+    float* v_s = q_s + (size_t)chunk * DP;  // [chunk][COLS]
+    float* s_s = v_s + (size_t)chunk * COLS;  // [chunk][2]: beta, g
     const int entry = blockIdx.z, head = blockIdx.y;
-    const int col0 = blockIdx.x * cols;
-    const int sub = threadIdx.x % lanes;
-    const int col = col0 + threadIdx.x / lanes;
+    const int col0 = blockIdx.x * COLS;
+    const int sub = threadIdx.x % LANES, colw = threadIdx.x / LANES;
+    const int col = col0 + colw;
     const bool live = col < dv;
     const int qk_head = head / qk_rep;
     const int first = q_start[entry], n = q_len[entry];
     float* S_col = state + (size_t)slots[entry] * state_stride + ((size_t)head * dv + (live ? col : 0)) * d;
 
+    // a lane's rows lie together: 16 bytes at a time where every column begins at a multiple of 16 bytes
+    const bool wide = (d & 3) == 0 && (state_stride & 3) == 0;
     float S[R];
 #pragma unroll
-    for (int i = 0; i < R; ++i) {
-        const int r = sub + i * lanes;
-        S[i] = (live && r < d) ? S_col[r] : 0.0f;
+    for (int i = 0; i < R; i += 4) {
+        const int r = sub * R + i;
+        if (wide) {
+            const float4 s4 = (live && r < d) ? *(const float4*)(S_col + r) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            S[i] = s4.x; S[i + 1] = s4.y; S[i + 2] = s4.z; S[i + 3] = s4.w;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) S[i + j] = (live && r + j < d) ? S_col[r + j] : 0.0f;
+        }
     }
     const float decay = MODE == 0 ? decays[head] : 0.0f;
+    float* o_col = o_raw + (size_t)head * dv + col;
+    const size_t o_stride = (size_t)heads * dv;
 
     for (int t0 = 0; t0 < n; t0 += chunk) {
         const int m = min(chunk, n - t0);
         __syncthreads();
-        for (int i = threadIdx.x; i < m * d; i += SCAN_THREADS) {
-            const int tt = i / d, r = i - tt * d;
-            const float* row = src + (size_t)(first + t0 + tt) * stride;
-            const float kv = row[k_at + qk_head * d + r], qv = row[q_at + qk_head * d + r];
-            k_s[tt * d + r] = MODE == 0 ? silu_f(kv) : kv;
-            q_s[tt * d + r] = MODE == 0 ? silu_f(qv) : qv;
+        for (int i = threadIdx.x; i < m * DP; i += SCAN_THREADS) {
+            const int tt = i / DP, r = i - tt * DP;
+            float kv = 0.0f, qv = 0.0f;
+            if (r < d) {
+                const float* row = src + (size_t)(first + t0 + tt) * stride;
+                kv = row[k_at + qk_head * d + r];
+                qv = row[q_at + qk_head * d + r];
+                if (MODE == 0) { kv = silu_f(kv); qv = silu_f(qv); }
+            }
+            k_s[i] = kv;
+            q_s[i] = qv;
         }
-        for (int i = threadIdx.x; i < m * cols; i += SCAN_THREADS) {
-            const int tt = i / cols, c = i - tt * cols;
+        for (int i = threadIdx.x; i < m * COLS; i += SCAN_THREADS) {
+            const int tt = i / COLS, c = i - tt * COLS;
             float vv = 0.0f;
             if (col0 + c < dv) {
                 vv = src[(size_t)(first + t0 + tt) * stride + v_at + head * dv + col0 + c];
                 if (MODE == 0) vv = silu_f(vv);
             }
-            v_s[tt * cols + c] = vv;
+            v_s[i] = vv;
         }
         if (MODE == 1)
             for (int i = threadIdx.x; i < m; i += SCAN_THREADS) {
@@ -85,104 +135,103 @@ matrix_scan_kernel(const float* __restrict__ src, int stride, int q_at, int k_at
                 s_s[2 * i + 1] = row[g_at + head];
             }
         __syncthreads();
-        for (int tt = 0; tt < m; ++tt) {
-            const float* kt = k_s + tt * d;
-            const float* qt = q_s + tt * d;
-            const float vv = v_s[tt * cols + threadIdx.x / lanes];
-            float acc = 0.0f;
-            if (MODE == 0) {
+        const float* kt = k_s + sub * R;
+        const float* qt = q_s + sub * R;
+        int tt = 0;
+        for (; tt + 4 <= m; tt += 4) {
+            float acc[4];
 #pragma unroll
-                for (int i = 0; i < R; ++i) {
-                    const int r = sub + i * lanes;
-                    if (r < d) {
-                        S[i] = fmaf(decay, S[i], kt[r] * vv);
-                        acc = fmaf(S[i], qt[r], acc);
-                    }
-                }
-            } else {
-                const float beta = s_s[2 * tt], g = s_s[2 * tt + 1];
-                float read = 0.0f;
+            for (int u = 0; u < 4; ++u)
+                acc[u] = scan_token<MODE, R, LANES>(S, kt + (tt + u) * DP, qt + (tt + u) * DP, v_s[(tt + u) * COLS + colw], decay,
+                                                    MODE == 1 ? s_s[2 * (tt + u)] : 0.0f, MODE == 1 ? s_s[2 * (tt + u) + 1] : 0.0f);
 #pragma unroll
-                for (int i = 0; i < R; ++i) {
-                    const int r = sub + i * lanes;
-                    if (r < d) {
-                        S[i] *= g;
-                        read = fmaf(S[i], kt[r], read);
-                    }
-                }
-                const float u = beta * (vv - column_sum(read, lanes));
+            for (int u = 0; u < 4; ++u) acc[u] = column_sum<LANES>(acc[u]);
+            if (live && sub == 0) {
 #pragma unroll
-                for (int i = 0; i < R; ++i) {
-                    const int r = sub + i * lanes;
-                    if (r < d) {
-                        S[i] = fmaf(kt[r], u, S[i]);
-                        acc = fmaf(S[i], qt[r], acc);
-                    }
-                }
+                for (int u = 0; u < 4; ++u) o_col[(size_t)(first + t0 + tt + u) * o_stride] = acc[u];
             }
-            acc = column_sum(acc, lanes);
-            if (live && sub == 0) o_raw[(size_t)(first + t0 + tt) * heads * dv + head * dv + col] = acc;
+        }
+        for (; tt < m; ++tt) {
+            float acc = scan_token<MODE, R, LANES>(S, kt + tt * DP, qt + tt * DP, v_s[tt * COLS + colw], decay,
+                                                   MODE == 1 ? s_s[2 * tt] : 0.0f, MODE == 1 ? s_s[2 * tt + 1] : 0.0f);
+            acc = column_sum<LANES>(acc);
+            if (live && sub == 0) o_col[(size_t)(first + t0 + tt) * o_stride] = acc;
         }
     }
     if (live) {
 #pragma unroll
-        for (int i = 0; i < R; ++i) {
-            const int r = sub + i * lanes;
-            if (r < d) S_col[r] = S[i];
+        for (int i = 0; i < R; i += 4) {
+            const int r = sub * R + i;
+            if (wide) {
+                if (r < d) *(float4*)(S_col + r) = make_float4(S[i], S[i + 1], S[i + 2], S[i + 3]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (r + j < d) S_col[r + j] = S[i + j];
+            }
         }
     }
 }
 
-// Lanes a column and tokens a chunk for key size d; false if d is out of range.
-static bool scan_shape(int d, int* lanes, int* rows, int* chunk) {
+// Lanes a column, rows a lane and tokens a chunk for key size d; false if d is out of range.
+static bool scan_shape(int d, int longest, int* lanes, int* rows, int* chunk) {
     if (d <= 0 || d > 1024) return false;
     *rows = d <= 512 ? 8 : 16;
     int l = 1;
     while (l * *rows < d) l <<= 1;
     *lanes = l;
-    int c = 4096 / d;
-    *chunk = c < 1 ? 1 : (c > 16 ? 16 : c);
+    int c = 6144 / (l * *rows);      // k and q of a chunk stay under 48 KB of LDS
+    *chunk = c < 1 ? 1 : (c > 32 ? 32 : c);
+    // no more LDS than the longest entry fills (single tokens: a few hundred bytes, so that many workgroups share a compute unit)
+    if (longest > 0 && longest < *chunk) *chunk = longest;
     return true;
 }
 
 template <int MODE>
 static int launch_scan(const float* src, int stride, int q_at, int k_at, int v_at, int beta_at, int g_at, const float* decays,
                        float* state, size_t state_stride, const int32_t* q_start, const int32_t* q_len, const int32_t* slots,
-                       float* o_raw, int entries, int heads, int qk_rep, int d, int dv, hipStream_t stream) {
+                       float* o_raw, int entries, int heads, int qk_rep, int d, int dv, int longest, hipStream_t stream) {
     int lanes, rows, chunk;
-    if (!scan_shape(d, &lanes, &rows, &chunk) || heads <= 0 || dv <= 0 || qk_rep <= 0 || heads % qk_rep) return -1;
+    if (!scan_shape(d, longest, &lanes, &rows, &chunk) || heads <= 0 || dv <= 0 || qk_rep <= 0 || heads % qk_rep) return -1;
     if (state_stride < (size_t)heads * d * dv) return -1;
     const int cols = SCAN_THREADS / lanes;
     dim3 grid((dv + cols - 1) / cols, heads, entries), block(SCAN_THREADS);
-    const size_t lds = ((size_t)2 * chunk * d + (size_t)chunk * cols + 2 * chunk) * sizeof(float);
-    if (rows == 8)
-        hipLaunchKernelGGL((matrix_scan_kernel<MODE, 8>), grid, block, lds, stream, src, stride, q_at, k_at, v_at, beta_at, g_at, decays,
-                           state, state_stride, q_start, q_len, slots, o_raw, heads, qk_rep, d, dv, lanes, chunk);
-    else
-        hipLaunchKernelGGL((matrix_scan_kernel<MODE, 16>), grid, block, lds, stream, src, stride, q_at, k_at, v_at, beta_at, g_at, decays,
-                           state, state_stride, q_start, q_len, slots, o_raw, heads, qk_rep, d, dv, lanes, chunk);
+    const size_t lds = ((size_t)2 * chunk * lanes * rows + (size_t)chunk * cols + 2 * chunk) * sizeof(float);
+#define KIPP_SCAN(R, L)                                                                                                        \
+    hipLaunchKernelGGL((matrix_scan_kernel<MODE, R, L>), grid, block, lds, stream, src, stride, q_at, k_at, v_at, beta_at, g_at, \
+                       decays, state, state_stride, q_start, q_len, slots, o_raw, heads, qk_rep, d, dv, chunk)
+    if (rows == 16) KIPP_SCAN(16, 64);
+    else if (lanes == 1) KIPP_SCAN(8, 1);
+    else if (lanes == 2) KIPP_SCAN(8, 2);
+    else if (lanes == 4) KIPP_SCAN(8, 4);
+    else if (lanes == 8) KIPP_SCAN(8, 8);
+    else if (lanes == 16) KIPP_SCAN(8, 16);
+    else if (lanes == 32) KIPP_SCAN(8, 32);
+    else KIPP_SCAN(8, 64);
+#undef KIPP_SCAN
     return KIPP_LAUNCH_CHECK();
 }
 
 // proj: float32 [tokens][stride], columns q [heads d] | k [heads d] | v [heads dv] | ... before their silu.
+// `longest`: the most tokens an entry brings, if the host knows (0: it does not); it only sizes the chunks.
 extern "C" int kipp_decay_scan(const float* proj, int stride, const float* decays, float* state, size_t state_stride,
                                const int32_t* q_start, const int32_t* q_len, const int32_t* slots, float* o_raw, int entries,
-                               int heads, int d, int dv, hipStream_t stream) {
+                               int heads, int d, int dv, int longest, hipStream_t stream) {
     if (entries <= 0) return 0;
     if (stride < 2 * heads * d + heads * dv) return -1;
     return launch_scan<0>(proj, stride, 0, heads * d, 2 * heads * d, 0, 0, decays, state, state_stride, q_start, q_len, slots, o_raw,
-                          entries, heads, 1, d, dv, stream);
+                          entries, heads, 1, d, dv, longest, stream);
 }
 
 // prep: float32 [tokens][stride], columns q [kv_heads d] | k [kv_heads d] | v [heads dv] | beta [heads] | g [heads], ready.
 extern "C" int kipp_delta_scan(const float* prep, int stride, float* state, size_t state_stride, const int32_t* q_start,
                                const int32_t* q_len, const int32_t* slots, float* o_raw, int entries, int heads, int kv_heads,
-                               int d, int dv, hipStream_t stream) {
+                               int d, int dv, int longest, hipStream_t stream) {
     if (entries <= 0) return 0;
     if (kv_heads <= 0 || heads % kv_heads || stride < 2 * kv_heads * d + heads * dv + 2 * heads) return -1;
     const int c = 2 * kv_heads * d + heads * dv;
     return launch_scan<1>(prep, stride, 0, kv_heads * d, 2 * kv_heads * d, c, c + heads, nullptr, state, state_stride, q_start, q_len,
-                          slots, o_raw, entries, heads, heads / kv_heads, d, dv, stream);
+                          slots, o_raw, entries, heads, heads / kv_heads, d, dv, longest, stream);
 }
 
 // One workgroup a token.  conv_w [channels][taps]; kept [slot][taps - 1][channels] at `kept_at` floats into the slot.

@@ -3,13 +3,13 @@
 //
 //     route    p = softmax(z) over all experts (float32); the `top` largest p (the lower index first among equals);
 //              weight = p / (sum of the chosen p + eps)
-//     sort     the (token, choice) pairs in runs of one expert each, cut into tiles of up to 16 (or 64) rows; the list of tiles
+//     sort     the (token, choice) pairs in runs of one expert each, cut into tiles of up to 16 (or 128) rows; the list of tiles
 //              is made on the device, so the host never learns the counts and the launches have a fixed shape
 //     expert   a tile's rows against its expert's matrix: out[row][n] = act(sum_k W_e[n][k] x[row][k]).  bfloat16 with K a
-//              multiple of 32: on the matrix cores, a workgroup a (tile of up to 64 rows, 256 columns), a wave 64 of the
-//              columns in 4 x 4 fragments of 16 x 16, operands straight from memory (a fragment row is 64 bytes of a
-//              matrix row); a tile of a few rows (single tokens) multiplies only the fragments it has, and is then bound
-//              by the read of its expert's matrix.  Else (float32, other K): a lane takes a column of a tile of 16 rows.
+//              multiple of 32: on the matrix cores, a workgroup a (tile of up to 128 rows, 256 columns), a wave 64 of the
+//              columns in 8 x 4 fragments of 16 x 16; steps of 64 numbers of k come from memory 128 bytes a row (eight
+//              lanes side by side) into registers while the step before is multiplied out of LDS; a tile of a few rows
+//              (single tokens) multiplies only the fragments it has, and is then bound by the read of its expert's matrix.  Else (float32, other K): a lane takes a column of a tile of 16 rows.
 //              Either way the sum over k runs in one order for every row, so a row's result does not depend on its tile
 //     combine  out[t] = sum_j weight[t][j] y[place of (t, j)] (+ the shared expert's result, slabs added in order)
 #include "common.h"
@@ -21,9 +21,12 @@
 #define TILE_ROWS 16
 #define EXPERT_COLS 256
 #define EXPERT_KC 128
-#define MFMA_ROWS 64        // rows of a tile of the matrix-core product: four fragments of 16
+#define MFMA_ROWS 128       // rows of a tile of the matrix-core product: eight fragments of 16
 #define MFMA_COLS 256       // columns of a workgroup: four waves with four fragments each
+#define MFMA_KC 64          // numbers of k a step brings into LDS
+#define MFMA_PITCH 72       // bfloat16 numbers from a row to the next in LDS
 #define MFMA_THREADS 256
+#define XCDS 8              // dies of the chip; consecutive workgroups of a launch go to them in turn
 
 enum { ACT_NONE = -1, ACT_SILU = 0, ACT_RELU = 1, ACT_GELU = 2, ACT_GELU_TANH = 3 };
 
@@ -197,62 +200,94 @@ template <typename TO>
 __global__ void __launch_bounds__(MFMA_THREADS)
 moe_expert_mfma_kernel(const bf16_t* __restrict__ x, const int32_t* __restrict__ gather, const bf16_t* __restrict__ w,
                        const int32_t* __restrict__ tiles, TO* __restrict__ out, int n_out, int k, int act) {
-    const int32_t* tile = tiles + (size_t)blockIdx.x * 3;
+    // 64 numbers of k of every row of the tile and of every column of the workgroup, a row 144 bytes apart from the next
+    // (the fragments' reads of 16 bytes a lane then spread over the banks)
+    __shared__ __attribute__((aligned(16))) bf16_t a_s[MFMA_ROWS * MFMA_PITCH];
+    __shared__ __attribute__((aligned(16))) bf16_t b_s[MFMA_COLS * MFMA_PITCH];
+    // Workgroups go to the chip's 8 dies in turn, each with an L2 of its own: the launch's workgroups are renumbered so
+    // that a die works on neighbouring tiles at a time, which are mostly row tiles of one expert and read the same
+    // columns of its matrix.
+    const unsigned launched = blockIdx.x + blockIdx.y * gridDim.x, total = gridDim.x * gridDim.y;
+    const unsigned die = launched % XCDS, turn = launched / XCDS, each = total / XCDS, more = total % XCDS;
+    const unsigned item = (die < more ? die * (each + 1) : more * (each + 1) + (die - more) * each) + turn;
+    const int32_t* tile = tiles + (size_t)(item % gridDim.x) * 3;
     const int rows = tile[2];
     if (rows == 0) return;      // uniform over the workgroup
     const int expert = tile[0], row0 = tile[1];
-    const int wave = threadIdx.x / KIPP_WAVE, lane = threadIdx.x & (KIPP_WAVE - 1), l16 = lane & 15, h = lane >> 4;
-    const int col0 = blockIdx.y * MFMA_COLS + wave * 64;
-    if (col0 >= n_out) return;  // uniform over the wave; the kernel has no barrier
+    const int tid = threadIdx.x;
+    const int wave = tid / KIPP_WAVE, lane = tid & (KIPP_WAVE - 1), l16 = lane & 15, h = lane >> 4;
+    const int col_base = (item / gridDim.x) * MFMA_COLS;
     const int mfrags = (rows + 15) >> 4;
-    const bf16_t* a_ptr[4];
-    const bf16_t* b_ptr[4];
+    // from memory, 8 threads take the 128 bytes of a row's step: thread t rows t / 8 + 32 i, bytes 16 (t % 8) ..
+    const int ld_row = tid >> 3, ld_ch = tid & 7;
+    // where a lane's rows begin, in numbers from x and from the expert's matrix (the launcher has checked that 32 bits hold them)
+    unsigned a_src[MFMA_ROWS / 32], b_src[MFMA_COLS / 32];
+    const bf16_t* w_e = w + (size_t)expert * n_out * k;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int r = min(16 * i + l16, rows - 1);          // rows beyond the tile's read its last one and are not stored
-        const size_t src = gather != nullptr ? (size_t)gather[row0 + r] : (size_t)(row0 + r);
-        a_ptr[i] = x + src * k + 8 * h;
-        const int c = min(col0 + 16 * i + l16, n_out - 1);
-        b_ptr[i] = w + ((size_t)expert * n_out + c) * k + 8 * h;
+    for (int i = 0; i < MFMA_ROWS / 32; ++i) {
+        const int r = min(ld_row + 32 * i, rows - 1);       // rows beyond the tile's read its last one and are not stored
+        const unsigned src = gather != nullptr ? (unsigned)gather[row0 + r] : (unsigned)(row0 + r);
+        a_src[i] = src * (unsigned)k + 8 * ld_ch;
     }
-    f32x4 acc[4][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < MFMA_COLS / 32; ++i) {
+        const int c = min(col_base + ld_row + 32 * i, n_out - 1);
+        b_src[i] = (unsigned)c * (unsigned)k + 8 * ld_ch;
+    }
+    u32x4 a_r[MFMA_ROWS / 32], b_r[MFMA_COLS / 32];
+    const u32x4 zero = (u32x4){0u, 0u, 0u, 0u};
+    auto fetch = [&](int k0) {
+        const bool there = k0 + 8 * ld_ch < k;              // k is a multiple of 32: the last step may be half a step
+#pragma unroll
+        for (int i = 0; i < MFMA_ROWS / 32; ++i)
+            if (32 * i < 16 * mfrags) a_r[i] = there ? *(const u32x4*)(x + a_src[i] + k0) : zero;
+#pragma unroll
+        for (int i = 0; i < MFMA_COLS / 32; ++i) b_r[i] = there ? *(const u32x4*)(w_e + b_src[i] + k0) : zero;
+    };
+    f32x4 acc[MFMA_ROWS / 16][4];
+#pragma unroll
+    for (int i = 0; i < MFMA_ROWS / 16; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
-    if (mfrags == 4) {
-#pragma unroll 2
-        for (int k0 = 0; k0 < k; k0 += 32) {
-            Frag a[4], b[4];
+    fetch(0);
+    for (int k0 = 0; k0 < k; k0 += MFMA_KC) {
+        __syncthreads();        // the step before has been multiplied
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                a[i].u = *(const u32x4*)(a_ptr[i] + k0);
-                b[i].u = *(const u32x4*)(b_ptr[i] + k0);
-            }
+        for (int i = 0; i < MFMA_ROWS / 32; ++i)
+            if (32 * i < 16 * mfrags) *(u32x4*)(a_s + (ld_row + 32 * i) * MFMA_PITCH + 8 * ld_ch) = a_r[i];
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < MFMA_COLS / 32; ++i) *(u32x4*)(b_s + (ld_row + 32 * i) * MFMA_PITCH + 8 * ld_ch) = b_r[i];
+        __syncthreads();
+        if (k0 + MFMA_KC < k) fetch(k0 + MFMA_KC);      // on its way while this step is multiplied
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i].v, b[j].v, acc[i][j], 0, 0, 0);
-        }
-    } else {
-#pragma unroll 2
-        for (int k0 = 0; k0 < k; k0 += 32) {
+        for (int half = 0; half < 2; ++half) {
             Frag b[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) b[j].u = *(const u32x4*)(b_ptr[j] + k0);
+            for (int j = 0; j < 4; ++j) b[j].u = *(const u32x4*)(b_s + (wave * 64 + 16 * j + l16) * MFMA_PITCH + 32 * half + 8 * h);
+            if (mfrags == MFMA_ROWS / 16) {          // a whole tile: nothing to ask between the fragments
 #pragma unroll
-            for (int i = 0; i < 3; ++i) {
-                if (i < mfrags) {
+                for (int i = 0; i < MFMA_ROWS / 16; ++i) {
                     Frag a;
-                    a.u = *(const u32x4*)(a_ptr[i] + k0);
+                    a.u = *(const u32x4*)(a_s + (16 * i + l16) * MFMA_PITCH + 32 * half + 8 * h);
 #pragma unroll
                     for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b[j].v, acc[i][j], 0, 0, 0);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < MFMA_ROWS / 16 - 1; ++i) {
+                    if (i < mfrags) {
+                        Frag a;
+                        a.u = *(const u32x4*)(a_s + (16 * i + l16) * MFMA_PITCH + 32 * half + 8 * h);
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b[j].v, acc[i][j], 0, 0, 0);
+                    }
                 }
             }
         }
     }
+    const int col0 = col_base + wave * 64;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < MFMA_ROWS / 16; ++i)
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const int r = 16 * i + 4 * h + v;
@@ -296,13 +331,15 @@ extern "C" int kipp_moe_route(const float* z, int parts, int stride, int32_t* ch
     return KIPP_LAUNCH_CHECK();
 }
 
-// `tile_rows`: the rows of the tiles that `kipp_moe_route` was asked for: 64 takes the matrix cores (bfloat16 x and w, K a multiple of 32), 16 the plain kernel.
+// `tile_rows`: the rows of the tiles that `kipp_moe_route` was asked for: 128 takes the matrix cores (bfloat16 x and w, K a multiple of 32), 16 the plain kernel.
 extern "C" int kipp_moe_expert(const void* x, int x_dtype, const int32_t* gather, const void* w, int w_dtype, const int32_t* tiles,
                                int max_tiles, void* out, int out_dtype, int n_out, int k, int act, int tile_rows, hipStream_t stream) {
     if (max_tiles <= 0) return 0;
     if (n_out <= 0 || k <= 0 || act < ACT_NONE || act > ACT_GELU_TANH) return -1;
     if (tile_rows == MFMA_ROWS) {
         if (x_dtype != KIPP_BF16 || w_dtype != KIPP_BF16 || k % 32) return -2;
+        // a lane's offsets into x and into an expert's matrix are 32 bits wide
+        if ((long long)max_tiles * MFMA_ROWS * k >= (1ll << 31) || (long long)n_out * k >= (1ll << 31)) return -2;
         dim3 grid(max_tiles, (n_out + MFMA_COLS - 1) / MFMA_COLS), block(MFMA_THREADS);
         if (out_dtype == KIPP_BF16)
             hipLaunchKernelGGL((moe_expert_mfma_kernel<bf16_t>), grid, block, 0, stream, (const bf16_t*)x, gather, (const bf16_t*)w, tiles,

@@ -637,17 +637,18 @@ def _scan_args(state, q_start, q_len, slots, o_raw, tokens, heads, d, dv, what):
 
 
 def decay_scan(proj: torch.Tensor, decays: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
-               slots: torch.Tensor, o_raw: torch.Tensor, heads: int, d: int, dv: int) -> torch.Tensor:
+               slots: torch.Tensor, o_raw: torch.Tensor, heads: int, d: int, dv: int, longest: int = 0) -> torch.Tensor:
     """Linear attention with a fixed decay a head over every entry's tokens, in order, from and into the entry's slot of
     `state` [slots, size] (float32, S as [head][column][row]).  `proj`: float32 [tokens, >= 2 heads d + heads dv], columns
-    q | k | v before their silu; `o_raw` float32 [tokens, heads dv] receives S^T q."""
+    q | k | v before their silu; `o_raw` float32 [tokens, heads dv] receives S^T q.  `longest`: the most tokens an entry
+    brings, if known (it sizes the kernel's chunks and changes no result)."""
     _dev(proj, decays, state, q_start, q_len, slots, o_raw)
     _need(proj.dim() == 2 and proj.dtype == torch.float32 and proj.shape[1] >= 2 * heads * d + heads * dv, "decay_scan: proj is float32 [tokens, q | k | v ...]")
     _need(decays.dtype == torch.float32 and decays.numel() == heads, "decay_scan: float32 decays [heads]")
     _scan_args(state, q_start, q_len, slots, o_raw, proj.shape[0], heads, d, dv, "decay_scan")
-    fn = _fn("linear_scan", "kipp_decay_scan", [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_size, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    fn = _fn("linear_scan", "kipp_decay_scan", [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_size, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(proj), proj.shape[1], _ptr(decays), _ptr(state), state.shape[1], _ptr(q_start), _ptr(q_len), _ptr(slots), _ptr(o_raw),
-              q_start.numel(), heads, d, dv, _stream()), "decay_scan")
+              q_start.numel(), heads, d, dv, max(0, int(longest)), _stream()), "decay_scan")
     return o_raw
 
 
@@ -686,16 +687,16 @@ def delta_prepare(proj: torch.Tensor, conv_w: torch.Tensor, a_log: torch.Tensor,
 
 
 def delta_scan(prep: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor, slots: torch.Tensor,
-               o_raw: torch.Tensor, heads: int, kv_heads: int, d: int, dv: int) -> torch.Tensor:
+               o_raw: torch.Tensor, heads: int, kv_heads: int, d: int, dv: int, longest: int = 0) -> torch.Tensor:
     """The gated delta rule over every entry's tokens, in order, from and into the entry's slot: S <- g S; u = beta (v - S^T k);
-    S <- S + k u^T; o = S^T q, with `prep` as `delta_prepare` leaves it."""
+    S <- S + k u^T; o = S^T q, with `prep` as `delta_prepare` leaves it.  `longest` as for `decay_scan`."""
     _dev(prep, state, q_start, q_len, slots, o_raw)
     _need(prep.dim() == 2 and prep.dtype == torch.float32 and prep.shape[1] >= 2 * kv_heads * d + heads * dv + 2 * heads and heads % kv_heads == 0,
           "delta_scan: prep is float32 [tokens, q | k | v | beta | g]")
     _scan_args(state, q_start, q_len, slots, o_raw, prep.shape[0], heads, d, dv, "delta_scan")
-    fn = _fn("linear_scan", "kipp_delta_scan", [_c_ptr, _c_int, _c_ptr, _c_size, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    fn = _fn("linear_scan", "kipp_delta_scan", [_c_ptr, _c_int, _c_ptr, _c_size, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(prep), prep.shape[1], _ptr(state), state.shape[1], _ptr(q_start), _ptr(q_len), _ptr(slots), _ptr(o_raw), q_start.numel(),
-              heads, kv_heads, d, dv, _stream()), "delta_scan")
+              heads, kv_heads, d, dv, max(0, int(longest)), _stream()), "delta_scan")
     return o_raw
 
 
@@ -717,11 +718,11 @@ def scan_finish(o_raw: torch.Tensor, gates: torch.Tensor, gate_at: int, norm_w: 
 
 ACTIVATIONS = {"silu": 0, "relu": 1, "gelu": 2, "gelu_tanh": 3}
 MOE_TILE_ROWS = 16
-MOE_MFMA_ROWS = 64     # rows of a tile of the experts' products on the matrix cores
+MOE_MFMA_ROWS = 128    # rows of a tile of the experts' products on the matrix cores
 
 
 def moe_tile_rows(dtype: torch.dtype, *contractions: int) -> int:
-    """Rows of the tiles that the experts' products take: 64 on the matrix cores (bfloat16, every contraction a multiple of
+    """Rows of the tiles that the experts' products take: 128 on the matrix cores (bfloat16, every contraction a multiple of
     32), else 16."""
     return MOE_MFMA_ROWS if dtype == torch.bfloat16 and all(k % 32 == 0 for k in contractions) else MOE_TILE_ROWS
 
@@ -755,7 +756,7 @@ def moe_route(z: torch.Tensor, experts: int, top: int, eps: float, chosen: torch
 def moe_expert(x: torch.Tensor, gather: Optional[torch.Tensor], w: torch.Tensor, tiles: torch.Tensor, out: torch.Tensor,
                activation: Optional[str] = None, tile_rows: int = 16) -> torch.Tensor:
     """Every tile's rows against its expert's matrix: out[row] = act(w[expert] x_row), x_row = x[gather[row]] (or x[row]);
-    `w` [experts, n_out, k], `out` [sorted rows, n_out].  `tile_rows`: what `moe_route` was given (64: the matrix cores)."""
+    `w` [experts, n_out, k], `out` [sorted rows, n_out].  `tile_rows`: what `moe_route` was given (128: the matrix cores)."""
     _dev(x, gather, w, tiles, out)
     _i32(tiles, "tiles")
     if gather is not None:
@@ -765,7 +766,7 @@ def moe_expert(x: torch.Tensor, gather: Optional[torch.Tensor], w: torch.Tensor,
     _need(out.shape[0] == (gather.numel() if gather is not None else x.shape[0]), "moe_expert: one output row a sorted row")
     _need(activation is None or activation in ACTIVATIONS, f"moe_expert: activation is one of {sorted(ACTIVATIONS)}")
     _need(tile_rows == MOE_TILE_ROWS or (tile_rows == MOE_MFMA_ROWS and x.dtype == torch.bfloat16 and w.shape[2] % 32 == 0),
-          "moe_expert: tiles of 16 rows, or of 64 for bfloat16 with K a multiple of 32")
+          "moe_expert: tiles of 16 rows, or of 128 for bfloat16 with K a multiple of 32")
     fn = _fn("moe", "kipp_moe_expert", [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(x), _code(x), _ptr(gather), _ptr(w), _code(w), _ptr(tiles), tiles.shape[0], _ptr(out), _code(out), w.shape[1], w.shape[2],
               -1 if activation is None else ACTIVATIONS[activation], int(tile_rows), _stream()), "moe_expert")

@@ -138,7 +138,7 @@ class RoutedMLP:
         weight = rt.empty((n, s.top), torch.float32)
         pair_token = torch.empty((pairs,), dtype=torch.int32, device=dev)
         place = torch.empty((pairs,), dtype=torch.int32, device=dev)
-        # bfloat16 experts whose two contractions are multiples of 32 run on the matrix cores, in tiles of 64 rows
+        # bfloat16 experts whose two contractions are multiples of 32 run on the matrix cores, in tiles of 128 rows
         tile_rows = ops.moe_tile_rows(self.w_up.dtype, s.hidden_size, s.expert_size)
         tiles = torch.empty((ops.moe_max_tiles(n, s.experts, s.top, tile_rows), 3), dtype=torch.int32, device=dev)
         ops.moe_route(z, s.experts, s.top, s.weight_eps, chosen, weight, pair_token, place, tiles, tile_rows=tile_rows)

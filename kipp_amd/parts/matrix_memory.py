@@ -77,7 +77,7 @@ class DecayAttention:
         hv = s.num_heads * s.v_head_dim
         proj = rt.linear(x, self.w_in)                    # float32 [n, q | k | v | gate]
         o_raw = rt.empty((n, hv), torch.float32)
-        ops.decay_scan(proj, self.decays, state, batch.q_start, batch.q_len, batch.slots, o_raw, s.num_heads, s.head_dim, s.v_head_dim)
+        ops.decay_scan(proj, self.decays, state, batch.q_start, batch.q_len, batch.slots, o_raw, s.num_heads, s.head_dim, s.v_head_dim, longest=batch.max_q_len)
         out = ops.scan_finish(o_raw, proj, 2 * s.num_heads * s.head_dim + hv, self.norm, s.norm_eps, "sigmoid", hv, rt.empty((n, hv), rt.act_dtype))
         return rt.linear(out, self.w_o, slabs=True, defer=True)
 
@@ -142,6 +142,6 @@ class GatedDelta:
         ops.delta_prepare(proj, self.conv, self.a_log, self.dt_bias, state, batch.seq_of_token, batch.q_start, batch.q_len, batch.slots, prep,
                           s.num_heads, s.num_kv_heads, s.head_dim, s.v_head_dim, channels + hv, channels + hv + s.num_heads, s.unit_eps)
         o_raw = rt.empty((n, hv), torch.float32)
-        ops.delta_scan(prep, state, batch.q_start, batch.q_len, batch.slots, o_raw, s.num_heads, s.num_kv_heads, s.head_dim, s.v_head_dim)
+        ops.delta_scan(prep, state, batch.q_start, batch.q_len, batch.slots, o_raw, s.num_heads, s.num_kv_heads, s.head_dim, s.v_head_dim, longest=batch.max_q_len)
         out = ops.scan_finish(o_raw, proj, channels, self.norm, s.norm_eps, "silu", s.v_head_dim, rt.empty((n, hv), rt.act_dtype))
         return rt.linear(out, self.w_o, slabs=True, defer=True)

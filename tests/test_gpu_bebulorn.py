@@ -286,8 +286,8 @@ def test_routed_feed_forward_kernels(dtype, experts, top, tokens, width, inner):
     pairs = tokens * top
     chosen, weight = torch.empty((tokens, top), dtype=torch.int32, device="cuda:0"), torch.empty((tokens, top), device="cuda:0")
     pair_token, place = torch.empty(pairs, dtype=torch.int32, device="cuda:0"), torch.empty(pairs, dtype=torch.int32, device="cuda:0")
-    tile_rows = ops.moe_tile_rows(ty, width, inner)       # 64 (the matrix cores) for bfloat16 where both contractions are multiples of 32
-    assert tile_rows == (64 if dtype == "bfloat16" and width % 32 == 0 and inner % 32 == 0 else 16)
+    tile_rows = ops.moe_tile_rows(ty, width, inner)       # 128 (the matrix cores) for bfloat16 where both contractions are multiples of 32
+    assert tile_rows == (128 if dtype == "bfloat16" and width % 32 == 0 and inner % 32 == 0 else 16)
     tiles = torch.full((ops.moe_max_tiles(tokens, experts, top, tile_rows), 3), -7, dtype=torch.int32, device="cuda:0")
     ops.moe_route(f32(z), experts, top, 1e-20, chosen, weight, pair_token, place, tiles, tile_rows=tile_rows)
     zz = z.astype(np.float64).sum(axis=0)[:, :experts]
