@@ -6,8 +6,8 @@
 //     sort     the (token, choice) pairs in runs of one expert each, cut into tiles of up to 16 (or 128) rows; the list of tiles
 //              is made on the device, so the host never learns the counts and the launches have a fixed shape
 //     expert   a tile's rows against its expert's matrix: out[row][n] = act(sum_k W_e[n][k] x[row][k]).  bfloat16 with K a
-//              multiple of 32: on the matrix cores, a workgroup a (tile of up to 128 rows, 256 columns), a wave 64 of the
-//              columns in 8 x 4 fragments of 16 x 16; steps of 64 numbers of k come from memory 128 bytes a row (eight
+//              multiple of 32: on the matrix cores, a workgroup a (tile of up to 128 rows, 128 columns), a wave 32 of the
+//              columns in 8 x 2 fragments of 16 x 16 (two workgroups share a compute unit's registers); steps of 64 numbers of k come from memory 128 bytes a row (eight
 //              lanes side by side) into registers while the step before is multiplied out of LDS; a tile of a few rows
 //              (single tokens) multiplies only the fragments it has, and is then bound by the read of its expert's matrix.  Else (float32, other K): a lane takes a column of a tile of 16 rows.
 //              Either way the sum over k runs in one order for every row, so a row's result does not depend on its tile
@@ -22,7 +22,8 @@
 #define EXPERT_COLS 256
 #define EXPERT_KC 128
 #define MFMA_ROWS 128       // rows of a tile of the matrix-core product: eight fragments of 16
-#define MFMA_COLS 256       // columns of a workgroup: four waves with four fragments each
+#define MFMA_COLS 128       // columns of a workgroup: four waves with two fragments each
+#define MFMA_NF (MFMA_COLS / 64)
 #define MFMA_KC 64          // numbers of k a step brings into LDS
 #define MFMA_PITCH 72       // bfloat16 numbers from a row to the next in LDS
 #define MFMA_THREADS 256
@@ -244,11 +245,11 @@ moe_expert_mfma_kernel(const bf16_t* __restrict__ x, const int32_t* __restrict__
 #pragma unroll
         for (int i = 0; i < MFMA_COLS / 32; ++i) b_r[i] = there ? *(const u32x4*)(w_e + b_src[i] + k0) : zero;
     };
-    f32x4 acc[MFMA_ROWS / 16][4];
+    f32x4 acc[MFMA_ROWS / 16][MFMA_NF];
 #pragma unroll
     for (int i = 0; i < MFMA_ROWS / 16; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+        for (int j = 0; j < MFMA_NF; ++j) acc[i][j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
     fetch(0);
     for (int k0 = 0; k0 < k; k0 += MFMA_KC) {
         __syncthreads();        // the step before has been multiplied
@@ -261,16 +262,16 @@ moe_expert_mfma_kernel(const bf16_t* __restrict__ x, const int32_t* __restrict__
         if (k0 + MFMA_KC < k) fetch(k0 + MFMA_KC);      // on its way while this step is multiplied
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
-            Frag b[4];
+            Frag b[MFMA_NF];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) b[j].u = *(const u32x4*)(b_s + (wave * 64 + 16 * j + l16) * MFMA_PITCH + 32 * half + 8 * h);
+            for (int j = 0; j < MFMA_NF; ++j) b[j].u = *(const u32x4*)(b_s + (wave * 16 * MFMA_NF + 16 * j + l16) * MFMA_PITCH + 32 * half + 8 * h);
             if (mfrags == MFMA_ROWS / 16) {          // a whole tile: nothing to ask between the fragments
 #pragma unroll
                 for (int i = 0; i < MFMA_ROWS / 16; ++i) {
                     Frag a;
                     a.u = *(const u32x4*)(a_s + (16 * i + l16) * MFMA_PITCH + 32 * half + 8 * h);
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b[j].v, acc[i][j], 0, 0, 0);
+                    for (int j = 0; j < MFMA_NF; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b[j].v, acc[i][j], 0, 0, 0);
                 }
             } else {
 #pragma unroll
@@ -279,13 +280,13 @@ moe_expert_mfma_kernel(const bf16_t* __restrict__ x, const int32_t* __restrict__
                         Frag a;
                         a.u = *(const u32x4*)(a_s + (16 * i + l16) * MFMA_PITCH + 32 * half + 8 * h);
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b[j].v, acc[i][j], 0, 0, 0);
+                        for (int j = 0; j < MFMA_NF; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b[j].v, acc[i][j], 0, 0, 0);
                     }
                 }
             }
         }
     }
-    const int col0 = col_base + wave * 64;
+    const int col0 = col_base + wave * 16 * MFMA_NF;
 #pragma unroll
     for (int i = 0; i < MFMA_ROWS / 16; ++i)
 #pragma unroll
@@ -294,7 +295,7 @@ moe_expert_mfma_kernel(const bf16_t* __restrict__ x, const int32_t* __restrict__
             if (r < rows) {
                 TO* dst = out + (size_t)(row0 + r) * n_out;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
+                for (int j = 0; j < MFMA_NF; ++j) {
                     const int c = col0 + 16 * j + l16;
                     if (c < n_out) store_f(dst, c, activate(acc[i][j][v], act));
                 }
