@@ -12,7 +12,7 @@ import os
 from dataclasses import dataclass
 from typing import Callable, Dict
 
-from .specs import (AttentionSpec, ConfigError, DecayAttentionSpec, EmbeddingSpec, GatedDeltaSpec, GatedMLPSpec,
+from .specs import (AttentionSpec, BandScaledRopeSpec, ParallelMixerSpec, SSDSpec, ConfigError, DecayAttentionSpec, EmbeddingSpec, GatedDeltaSpec, GatedMLPSpec,
                     HeadSpec, HyperConnectionSpec, LatentAttentionSpec, LayerNormSpec, LayerRun, LayerSpec, MLSTMSpec,
                     MixedHeadAttentionSpec, ModelSpec, NoPositionSpec, OnePlusRMSNormSpec, RMSNormSpec, RopeSpec,
                     RoutedMLPSpec, ScaledRopeSpec)
@@ -109,3 +109,8 @@ from . import bebulorn as _bebulorn  # noqa: E402
 
 register_architecture(_bebulorn.ARCHITECTURE, _bebulorn.BebulornConfig.from_dict)
 BebulornConfig = _bebulorn.BebulornConfig
+
+from . import zivazen as _zivazen  # noqa: E402
+
+register_architecture(_zivazen.ARCHITECTURE, _zivazen.ZivazenConfig.from_dict)
+ZivazenConfig = _zivazen.ZivazenConfig

@@ -107,6 +107,34 @@ class ScaledRopeSpec:
 
 
 @dataclass(frozen=True)
+class BandScaledRopeSpec:
+    """Rotary position encoding whose slow frequencies are divided by `factor`, by wavelength bands: with f_i =
+    theta^(-2i / rotary_dim) and wavelength l_i = 2 pi / f_i, f_i is kept where l_i < original / high, divided by `factor`
+    where l_i > original / low, and between the two blended, s = (original / l_i - low) / (high - low):
+    (1 - s) f_i / factor + s f_i.  Cosines and sines keep their size."""
+    head_dim: int
+    theta: float
+    factor: float
+    low: float
+    high: float
+    original: float
+    rotary_dim: Optional[int] = None
+    pairing: str = "half"
+    kind: str = "rope_band_scaled"
+
+    def __post_init__(self):
+        rd = self.head_dim if self.rotary_dim is None else self.rotary_dim
+        if rd <= 0 or rd % 2 or rd > self.head_dim:
+            raise ConfigError(f"rotary_dim {rd} must be even and in (0, head_dim={self.head_dim}]")
+        if not self.theta > 0:
+            raise ConfigError(f"rope theta must be positive, got {self.theta}")
+        if not (self.factor > 0 and self.original > 0 and self.low > 0 and self.high > 0) or self.low == self.high:
+            raise ConfigError("rope scaling: factor, original, low and high must be positive, low and high different")
+        if self.pairing not in ("half", "interleaved"):
+            raise ConfigError(f"rope pairing {self.pairing!r} is not one of half, interleaved")
+
+
+@dataclass(frozen=True)
 class NoPositionSpec:
     """No position encoding inside the mixer."""
     kind: str = "none"
@@ -131,6 +159,12 @@ class AttentionSpec:
     `softcap` c: a score s (scale and head factor applied) becomes c tanh(s / c) before the softmax.
     `head_temp` name: a tensor [heads] of that local name multiplies the scores of each query head.
     `v_norm_eps`: every head of a value is divided by its root mean square (no weight) before it is cached.
+    `chunk` C (instead of a window): position i sees j <= i only when floor(i / C) = floor(j / C), chunks counted from
+    position 0 of the sequence.  `sink`: one is added to the softmax's denominator (a key of score 0 without a value).
+    `out_bias` name: the output projection has a bias of that local name.  `v_mix`: "source": this run's values (before
+    any mixing) are what later runs of the same step mix in; "mix": v <- (1 - lambda) v + lambda v_source before it is
+    cached, lambda the one number of the tensor `v_mix_name`, v_source the source run's values of the same token (a
+    source declares the tensor too and leaves it unused).
     """
     hidden_size: int
     num_heads: int
@@ -153,10 +187,21 @@ class AttentionSpec:
     softcap: Optional[float] = None
     head_temp: Optional[str] = None
     v_norm_eps: Optional[float] = None
+    chunk: Optional[int] = None
+    sink: bool = False
+    out_bias: Optional[str] = None
+    v_mix: Optional[str] = None
+    v_mix_name: str = "vmix"
 
     def __post_init__(self):
         if self.num_heads <= 0 or self.num_kv_heads <= 0:
             raise ConfigError("attention needs at least one query head and one key/value head")
+        if self.chunk is not None and (self.chunk <= 0 or self.window is not None):
+            raise ConfigError("attention chunk must be positive and stands instead of a window")
+        if self.v_mix not in (None, "source", "mix"):
+            raise ConfigError(f"attention v_mix {self.v_mix!r} is not one of source, mix")
+        if self.v_mix is not None and not self.own_kv:
+            raise ConfigError("attention v_mix needs values of the mixer's own")
         if self.softcap is not None and not self.softcap > 0:
             raise ConfigError(f"attention softcap must be positive, got {self.softcap}")
         if self.v_norm_eps is not None and not self.v_norm_eps >= 0:
@@ -205,7 +250,8 @@ class AttentionSpec:
     def plain(self) -> bool:
         """None of the extras: the mixer's first kernels (weighted norm, rotation, fused decode) apply."""
         return not self.bias and self.qk_norm_weight and self.q_temp is None and self.v_head_dim is None and self.own_kv \
-            and self.softcap is None and self.head_temp is None and self.v_norm_eps is None
+            and self.softcap is None and self.head_temp is None and self.v_norm_eps is None \
+            and self.chunk is None and not self.sink and self.v_mix is None
 
 
 @dataclass(frozen=True)
@@ -352,6 +398,67 @@ class GatedDeltaSpec:
 
 
 @dataclass(frozen=True)
+class SSDSpec:
+    """A selective state space layer in its dual form (Mamba-2): per head a state S [state_size, head_dim] that starts at
+    zero and is carried from token to token in float32, beside the last `conv_taps` - 1 inputs of the short convolution.
+
+    W_in x = [z | u | B | C | dt] (z, u of num_heads head_dim numbers, B, C of groups state_size, dt of num_heads); u, B and
+    C pass a causal filter a channel over their last `conv_taps` inputs (with a bias; zeros before the start, the last tap
+    is the current token's) and silu; dt = softplus(dt + dt_bias).  Head h reads B and C of group h // (num_heads / groups):
+    S <- exp(-exp(A_h) dt) S + dt B u^T;  y = S^T C + D_h u.  y times silu(z), then an RMS norm in `norm_groups` equal
+    parts (`norm_eps`) times the norm weight, then W_o.
+    `names`: local tensor names of (in, conv, conv bias, dt_bias, A, D, norm, o)."""
+    hidden_size: int
+    num_heads: int
+    head_dim: int
+    state_size: int
+    groups: int
+    conv_taps: int
+    norm_groups: int
+    norm_eps: float
+    prefix: str = ""
+    kind: str = "ssd"
+    names: Tuple[str, ...] = ("in", "conv", "conv.b", "dt_bias", "A_log", "D", "norm", "o")
+
+    def __post_init__(self):
+        if self.num_heads <= 0 or self.groups <= 0 or self.num_heads % self.groups or self.num_heads > 1024:
+            raise ConfigError(f"ssd: heads {self.num_heads} must be a positive multiple of groups {self.groups}, up to 1,024")
+        if self.head_dim <= 0 or not 0 < self.state_size <= 1024:
+            raise ConfigError("ssd: head size must be positive, state size from 1 to 1,024")
+        if not 1 <= self.conv_taps <= 16:
+            raise ConfigError(f"ssd: the short convolution takes 1 to 16 taps, got {self.conv_taps}")
+        if self.norm_groups <= 0 or self.inner % self.norm_groups:
+            raise ConfigError(f"ssd: norm_groups {self.norm_groups} must divide heads * head size {self.inner}")
+        if len(self.names) != 8:
+            raise ConfigError("names: eight local tensor names")
+
+    @property
+    def inner(self) -> int:
+        return self.num_heads * self.head_dim
+
+    @property
+    def channels(self) -> int:
+        """Channels that pass the short convolution: u | B | C."""
+        return self.inner + 2 * self.groups * self.state_size
+
+    @property
+    def in_dim(self) -> int:
+        return self.inner + self.channels + self.num_heads
+
+
+@dataclass(frozen=True)
+class ParallelMixerSpec:
+    """Two mixers side by side that read the same input: delta = left_scale * left(x) + right_scale * right(x).  At most one
+    of them keeps keys and values in pages and at most one keeps state of fixed size."""
+    left: object
+    right: object
+    left_scale: float = 1.0
+    right_scale: float = 1.0
+    prefix: str = ""
+    kind: str = "parallel_mixer"
+
+
+@dataclass(frozen=True)
 class HyperConnectionSpec:
     """How one sublayer reads from and writes to `streams` copies of the residual stream: it reads sum_r in[r] X_r and
     its result y goes back as X_t <- sum_r mix[r, t] X_r + out[t] y for every t at once.  `learned` False: no tensors,
@@ -433,13 +540,15 @@ class MixedHeadAttentionSpec:
 
 @dataclass(frozen=True)
 class GatedMLPSpec:
-    """down(act(gate(x)) * up(x)); `activation` is "silu" or "relu".  `names`: the local tensor names of (gate, up, down)."""
+    """down(act(gate(x)) * up(x)); `activation` is "silu" or "relu".  `names`: the local tensor names of (gate, up, down);
+    `bias_names`: those of their biases (None: the projections have none)."""
     hidden_size: int
     intermediate_size: int
     activation: str = "silu"
     prefix: str = ""
     kind: str = "gated_mlp"
     names: Tuple[str, str, str] = ("gate_proj.weight", "up_proj.weight", "down_proj.weight")
+    bias_names: Optional[Tuple[str, str, str]] = None
 
     def __post_init__(self):
         if self.intermediate_size <= 0:
@@ -451,10 +560,14 @@ class GatedMLPSpec:
 @dataclass(frozen=True)
 class RoutedMLPSpec:
     """A mixture of `experts` small feed-forwards, of which a token uses `top`: W_down_e act(W_up_e x), `activation`
-    "gelu" (the exact one, with erf), "gelu_tanh", "silu" or "relu".  p = softmax(W_router x) over all experts in float32; the
+    "gelu" (the exact one, with erf), "gelu_tanh", "silu", "relu" or "relu2".  p = softmax(W_router x) over all experts in float32; the
     `top` largest are chosen (the lower index first among equals) and weigh their experts' results by p / (sum of the
     chosen p + `weight_eps`).  `shared_size` I: one more expert of inner size I (tensors under `shared_prefix`) runs for
-    every token and is added (None: none).  Expert e's tensors are `expert_prefix.format(e)` + (up, down)."""
+    every token and is added (None: none).  Expert e's tensors are `expert_prefix.format(e)` + (up, down).
+    `activation` "relu2" is the square of relu.  `router` "sigmoid": scores s = sigmoid(W_router x); the choice goes by
+    s + the tensor `correction_name` (None: no correction); with `groups` (count, keep) the experts form `count` equal groups
+    of neighbours, a group's score is the sum of its two largest choice scores, and only experts of the `keep` best groups can
+    be chosen; weights are s / (sum of the chosen s + `weight_eps`) * `route_scale`."""
     hidden_size: int
     experts: int
     top: int
@@ -468,16 +581,29 @@ class RoutedMLPSpec:
     expert_prefix: str = "e{}."
     shared_prefix: str = "shared."
     names: Tuple[str, str] = ("up", "down")
+    router: str = "softmax"
+    correction_name: Optional[str] = None
+    groups: Optional[Tuple[int, int]] = None
+    route_scale: float = 1.0
 
     def __post_init__(self):
+        if self.router not in ("softmax", "sigmoid"):
+            raise ConfigError(f"routed feed-forward: router {self.router!r} is not one of softmax, sigmoid")
+        if self.router == "softmax" and (self.correction_name is not None or self.groups is not None or self.route_scale != 1.0):
+            raise ConfigError("routed feed-forward: a correction, groups and a scale belong to the sigmoid router")
+        if self.groups is not None:
+            count, keep = self.groups
+            if count <= 0 or self.experts % count or not 0 < keep <= count or self.top > keep * (self.experts // count):
+                raise ConfigError(f"routed feed-forward: groups {self.groups}: equal groups of the {self.experts} experts, of which "
+                                  f"1 to count stay, with experts enough for the {self.top} a token uses")
         if not 0 < self.top <= self.experts:
             raise ConfigError(f"routed feed-forward: top {self.top} must be from 1 to experts {self.experts}")
         if self.experts > 1024 or self.top > 32:
             raise ConfigError("routed feed-forward: up to 1,024 experts, up to 32 a token")
         if self.expert_size <= 0 or (self.shared_size is not None and self.shared_size <= 0):
             raise ConfigError("routed feed-forward: inner sizes must be positive")
-        if self.activation not in ("gelu", "gelu_tanh", "silu", "relu"):
-            raise ConfigError(f"activation {self.activation!r} unsupported (gelu, gelu_tanh, silu, relu)")
+        if self.activation not in ("gelu", "gelu_tanh", "silu", "relu", "relu2"):
+            raise ConfigError(f"activation {self.activation!r} unsupported (gelu, gelu_tanh, silu, relu, relu2)")
 
 
 @dataclass(frozen=True)
@@ -493,7 +619,8 @@ class LayerSpec:
     ffn_norm, ffn_hc, ffn (the *_hc parts say how a sublayer reads and writes the copies);
     "hyper_pre_norm_mixer" is its first half alone.  "sandwich_norm" norms a sublayer's input and its result:
     x += a mixer_post_norm(mixer(mixer_norm(x))); x += a ffn_post_norm(ffn(ffn_norm(x))), a = `residual_scale`;
-    "sandwich_norm_mixer" is its first half alone.
+    "sandwich_norm_mixer" is its first half alone.  "parallel" has the roles mixer_norm, mixer and ffn: one norm whose
+    output both sublayers read, h = mixer_norm(x); x += mixer(h) + ffn(h); "parallel_mixer" is the same without a feed-forward.
     """
     parts: Tuple[Tuple[str, object], ...]
     block: str = "pre_norm"
@@ -558,6 +685,7 @@ class ModelSpec:
     stop_tokens: Tuple[int, ...] = field(default_factory=tuple)
     input_position: Optional[object] = None   # a position part applied to the residual stream after the embedding (None: none)
     streams: Optional[int] = None             # copies of the residual stream (None: one row a token; every layer is then no "hyper" block)
+    embedding_norm: Optional[object] = None   # a norm part applied to the embedding's rows before the first layer (None: none)
 
     def __post_init__(self):
         hyper = [layer.block.startswith("hyper_") for layer in self.layers]

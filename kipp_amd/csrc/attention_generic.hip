@@ -6,8 +6,9 @@
 // float32 path's kernel and the fallback of sizes the MFMA kernels refuse.
 //
 // For query position p of a sequence the keys are s in [max(0, p-window+1), p]
-// (window 0: from 0), score = (q . k_s) * scale (with `softcap` c > 0: c tanh(score / c)), softmax with the maximum
-// subtracted, out = sum p_s v_s  (/root/reference/src/kipp.c:2882-2922).  Keys are
+// (window 0: from 0; with `chunk` c > 0 from p - p % c, the start of p's chunk of c positions counted from 0), score = (q . k_s) * scale (with `softcap` c > 0: c tanh(score / c)), softmax with the maximum
+// subtracted (with `sink` one more term e^0 joins the denominator: a key of score 0 without a value),
+// out = sum p_s v_s  (/root/reference/src/kipp.c:2882-2922).  Keys are
 // taken in tiles of 64 aligned to absolute key index, so the sequence of
 // operations for one query depends on its own position only, never on what
 // else is in the batch.
@@ -57,7 +58,7 @@ __global__ void paged_attention_generic_kernel(
     const TQ* __restrict__ q, const TC* __restrict__ k_cache, const TC* __restrict__ v_cache, TO* __restrict__ out,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_of_token,
     const int32_t* __restrict__ block_table, int max_blocks,
-    int n_q, int n_kv, int d, int dv, int v_row, int page, float scale, int window, float softcap) {
+    int n_q, int n_kv, int d, int dv, int v_row, int page, float scale, int window, float softcap, int chunk, int sink) {
     __shared__ float q_s[HEADS_PER_BLOCK][MAX_D];
     __shared__ float p_s[HEADS_PER_BLOCK][KIPP_WAVE];
     __shared__ unsigned long long off_s[HEADS_PER_BLOCK][KIPP_WAVE];
@@ -71,7 +72,7 @@ __global__ void paged_attention_generic_kernel(
     const int pos = positions[t];
     const int seq = seq_of_token[t];
     const int32_t* table = block_table + (size_t)seq * max_blocks;
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int lo = chunk > 0 ? pos - pos % chunk : (window > 0 ? max(0, pos - window + 1) : 0);
 
     const TQ* q_row = q + ((size_t)t * n_q + head) * d;
     for (int e = lane; e < d; e += KIPP_WAVE) q_s[wave][e] = load_f(q_row, e);
@@ -122,6 +123,7 @@ __global__ void paged_attention_generic_kernel(
     }
     if (!active) return;
     TO* o_row = out + ((size_t)t * n_q + head) * dv;
+    if (sink) l += expf(-m);        // the term of score 0 (m is finite: a position sees itself)
     const float inv = 1.0f / l;
 #pragma unroll
     for (int c = 0; c < MAX_D / KIPP_WAVE; ++c) {
@@ -131,23 +133,34 @@ __global__ void paged_attention_generic_kernel(
 }
 
 // Values of width dv in rows of v_row numbers (v_row = dv for a value cache of its own).
-extern "C" int kipp_paged_attention_generic_capped(
+extern "C" int kipp_paged_attention_generic_masked(
     const void* q, int q_dtype, const void* k_cache, const void* v_cache, int cache_dtype, void* out, int out_dtype,
     const int32_t* positions, const int32_t* seq_of_token, const int32_t* block_table, int max_blocks,
     int n_tokens, int n_q, int n_kv, int d, int dv, int v_row, int page, float scale, int window, float softcap,
-    hipStream_t stream) {
+    int chunk, int sink, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
+    if (chunk < 0 || (chunk > 0 && window > 0)) return -1;
     if (d > MAX_D || d <= 0 || dv > MAX_D || dv <= 0 || v_row < dv || n_kv <= 0 || n_q % n_kv) return -1;
     dim3 grid((n_q + HEADS_PER_BLOCK - 1) / HEADS_PER_BLOCK, n_tokens), block(HEADS_PER_BLOCK * KIPP_WAVE);
 #define KIPP_PA(TQ, TC, TO)                                                                                    \
     hipLaunchKernelGGL((paged_attention_generic_kernel<TQ, TC, TO>), grid, block, 0, stream, (const TQ*)q,     \
                        (const TC*)k_cache, (const TC*)v_cache, (TO*)out, positions, seq_of_token, block_table, \
-                       max_blocks, n_q, n_kv, d, dv, v_row, page, scale, window, softcap)
+                       max_blocks, n_q, n_kv, d, dv, v_row, page, scale, window, softcap, chunk, sink)
     if (q_dtype == KIPP_F32 && cache_dtype == KIPP_F32 && out_dtype == KIPP_F32) KIPP_PA(float, float, float);
     else if (q_dtype == KIPP_BF16 && cache_dtype == KIPP_BF16 && out_dtype == KIPP_BF16) KIPP_PA(bf16_t, bf16_t, bf16_t);
     else return -2;
 #undef KIPP_PA
     return KIPP_LAUNCH_CHECK();
+}
+
+extern "C" int kipp_paged_attention_generic_capped(
+    const void* q, int q_dtype, const void* k_cache, const void* v_cache, int cache_dtype, void* out, int out_dtype,
+    const int32_t* positions, const int32_t* seq_of_token, const int32_t* block_table, int max_blocks,
+    int n_tokens, int n_q, int n_kv, int d, int dv, int v_row, int page, float scale, int window, float softcap,
+    hipStream_t stream) {
+    return kipp_paged_attention_generic_masked(q, q_dtype, k_cache, v_cache, cache_dtype, out, out_dtype, positions, seq_of_token,
+                                               block_table, max_blocks, n_tokens, n_q, n_kv, d, dv, v_row, page, scale, window, softcap,
+                                               0, 0, stream);
 }
 
 extern "C" int kipp_paged_attention_generic_v(

@@ -422,6 +422,19 @@ __global__ void scale_values_kernel(float* __restrict__ x, float s, size_t n) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) x[i] *= s;
 }
 
+// x[r][c] += scale * (sum of the slabs of delta[r][c]) + bias[c]: one term of a weighted sum of deltas, with the bias of
+// the product that made it (or none).
+__global__ void residual_add_scaled_kernel(float* __restrict__ x, const float* __restrict__ delta, size_t n, int parts, float scale,
+                                           const float* __restrict__ bias, int width) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        float d = delta[i];
+        for (int p = 1; p < parts; ++p) d += delta[p * n + i];
+        if (bias != nullptr) d += bias[i % width];
+        x[i] = fmaf(scale, d, x[i]);
+    }
+}
+
 extern "C" {
 
 int kipp_embed(const void* table, int table_dtype, const int32_t* tokens, float* out,
@@ -589,6 +602,15 @@ int kipp_scale_values(float* x, float s, size_t n, hipStream_t stream) {
     if (n == 0) return 0;
     const unsigned blocks = (unsigned)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
     hipLaunchKernelGGL(scale_values_kernel, dim3(blocks), dim3(256), 0, stream, x, s, n);
+    return KIPP_LAUNCH_CHECK();
+}
+
+int kipp_residual_add_scaled(float* x, const float* delta, int parts, size_t n, float scale, const float* bias, int width,
+                             hipStream_t stream) {
+    if (n == 0) return 0;
+    if (parts <= 0 || width <= 0 || n % width) return -1;
+    hipLaunchKernelGGL(residual_add_scaled_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x, delta, n, parts, scale, bias,
+                       width);
     return KIPP_LAUNCH_CHECK();
 }
 

@@ -1,8 +1,11 @@
 // Recurrent mixers whose memory is a matrix S [d, dv] a head, carried from token to token in float32 in the
-// request's slot: linear attention with a fixed decay a head, and the gated delta rule.
+// request's slot: linear attention with a fixed decay a head, the gated delta rule, and the selective state space
+// recurrence in its dual form (a decay a token and head).
 //
 //     decay   S <- a_h S + k v^T;                               o = S^T q      (q, k, v = silu of the projections)
 //     delta   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q      (q, k, v, beta, g made ready by `prepare`)
+//     gated   S <- g S + k v^T;                                 o = S^T q      (q, k, v, g made ready by `ssd_prepare`:
+//             k = B, q = C, v = dt x, g = exp(-exp(A_h) dt), dt = softplus(. + dt_bias))
 //
 // `scan`: a workgroup takes (entry, head, a run of columns of S) and walks the entry's tokens in order.  A column of S is
 // shared by L lanes side by side in a wave (L a power of two, 8 or 16 rows in a run a lane), so the sums over rows end in
@@ -38,10 +41,11 @@ __device__ __forceinline__ float scan_token(float (&S)[R], const float* __restri
         q[i] = q4.x; q[i + 1] = q4.y; q[i + 2] = q4.z; q[i + 3] = q4.w;
     }
     float acc = 0.0f;
-    if (MODE == 0) {
+    if (MODE == 0 || MODE == 2) {
+        const float a = MODE == 2 ? g : decay;
 #pragma unroll
         for (int i = 0; i < R; ++i) {
-            S[i] = fmaf(decay, S[i], k[i] * vv);
+            S[i] = fmaf(a, S[i], k[i] * vv);
             acc = fmaf(S[i], q[i], acc);
         }
     } else {
@@ -61,7 +65,8 @@ __device__ __forceinline__ float scan_token(float (&S)[R], const float* __restri
     return acc;
 }
 
-// MODE 0: fixed decay, inputs through silu.  MODE 1: delta rule, inputs as they are.  A column of S is shared by LANES
+// MODE 0: fixed decay, inputs through silu.  MODE 1: delta rule, inputs as they are.  MODE 2: a decay a token, inputs as
+// they are.  A column of S is shared by LANES
 // lanes side by side, lane `sub` with the R rows sub R .. sub R + R - 1 (read from LDS 16 bytes at a time; rows beyond d
 // are zeros there and stay zeros in S).
 template <int MODE, int R, int LANES>
@@ -128,10 +133,10 @@ matrix_scan_kernel(const float* __restrict__ src, int stride, int q_at, int k_at
             }
             v_s[i] = vv;
         }
-        if (MODE == 1)
+        if (MODE >= 1)
             for (int i = threadIdx.x; i < m; i += SCAN_THREADS) {
                 const float* row = src + (size_t)(first + t0 + i) * stride;
-                s_s[2 * i] = row[beta_at + head];
+                s_s[2 * i] = MODE == 1 ? row[beta_at + head] : 0.0f;
                 s_s[2 * i + 1] = row[g_at + head];
             }
         __syncthreads();
@@ -143,7 +148,7 @@ matrix_scan_kernel(const float* __restrict__ src, int stride, int q_at, int k_at
 #pragma unroll
             for (int u = 0; u < 4; ++u)
                 acc[u] = scan_token<MODE, R, LANES>(S, kt + (tt + u) * DP, qt + (tt + u) * DP, v_s[(tt + u) * COLS + colw], decay,
-                                                    MODE == 1 ? s_s[2 * (tt + u)] : 0.0f, MODE == 1 ? s_s[2 * (tt + u) + 1] : 0.0f);
+                                                    MODE >= 1 ? s_s[2 * (tt + u)] : 0.0f, MODE >= 1 ? s_s[2 * (tt + u) + 1] : 0.0f);
 #pragma unroll
             for (int u = 0; u < 4; ++u) acc[u] = column_sum<LANES>(acc[u]);
             if (live && sub == 0) {
@@ -153,7 +158,7 @@ matrix_scan_kernel(const float* __restrict__ src, int stride, int q_at, int k_at
         }
         for (; tt < m; ++tt) {
             float acc = scan_token<MODE, R, LANES>(S, kt + tt * DP, qt + tt * DP, v_s[tt * COLS + colw], decay,
-                                                   MODE == 1 ? s_s[2 * tt] : 0.0f, MODE == 1 ? s_s[2 * tt + 1] : 0.0f);
+                                                   MODE >= 1 ? s_s[2 * tt] : 0.0f, MODE >= 1 ? s_s[2 * tt + 1] : 0.0f);
             acc = column_sum<LANES>(acc);
             if (live && sub == 0) o_col[(size_t)(first + t0 + tt) * o_stride] = acc;
         }
@@ -311,6 +316,120 @@ extern "C" int kipp_delta_prepare(const float* proj, int stride, const float* co
     if (taps > 1)
         hipLaunchKernelGGL(conv_keep_kernel, dim3((channels + 255) / 256, entries), dim3(256), 0, stream, proj, stride, taps, state,
                            state_stride, kept_at, q_start, q_len, slots, channels);
+    return KIPP_LAUNCH_CHECK();
+}
+
+// prep: float32 [tokens][stride], columns q = C [groups n] | k = B [groups n] | v = dt x [heads p] | x [heads p] | g [heads], ready.
+extern "C" int kipp_gated_scan(const float* prep, int stride, float* state, size_t state_stride, const int32_t* q_start,
+                               const int32_t* q_len, const int32_t* slots, float* o_raw, int entries, int heads, int groups,
+                               int n, int p, int longest, hipStream_t stream) {
+    if (entries <= 0) return 0;
+    if (groups <= 0 || heads % groups || stride < 2 * groups * n + 2 * heads * p + heads) return -1;
+    return launch_scan<2>(prep, stride, 0, groups * n, 2 * groups * n, 0, 2 * groups * n + 2 * heads * p, nullptr, state, state_stride,
+                          q_start, q_len, slots, o_raw, entries, heads, heads / groups, n, p, longest, stream);
+}
+
+#define SSD_MAX_HEADS 1024
+
+// One workgroup a token.  proj: [z: inner | x: inner | B: groups n | C: groups n | dt: heads] (inner = heads p); the
+// channels x | B | C pass a causal filter (conv_w [channels][taps] with conv_b [channels], the slot's kept inputs ahead of a
+// portion; kept [taps - 1][channels] at `kept_at` floats into the slot) and silu.  prep as `kipp_gated_scan` reads it.
+__global__ void __launch_bounds__(SCAN_THREADS)
+ssd_prepare_kernel(const float* __restrict__ proj, int stride, const float* __restrict__ conv_w, const float* __restrict__ conv_b, int taps,
+                   const float* __restrict__ a_log, const float* __restrict__ dt_bias, const float* __restrict__ state,
+                   size_t state_stride, size_t kept_at, const int32_t* __restrict__ seq_of_token,
+                   const int32_t* __restrict__ q_start, const int32_t* __restrict__ slots, float* __restrict__ prep,
+                   int prep_stride, int heads, int groups, int n, int p) {
+    __shared__ float dt_s[SSD_MAX_HEADS];
+    const int t = blockIdx.x;
+    const int entry = seq_of_token[t];
+    const int first = q_start[entry];
+    const int inner = heads * p, gn = groups * n;
+    const int channels = inner + 2 * gn;
+    const float* kept = state + (size_t)slots[entry] * state_stride + kept_at;
+    const float* row = proj + (size_t)t * stride;
+    float* dst = prep + (size_t)t * prep_stride;
+    for (int h = threadIdx.x; h < heads; h += SCAN_THREADS) {
+        const float dt = softplus_f(row[2 * inner + 2 * gn + h] + dt_bias[h]);
+        dt_s[h] = dt;
+        dst[2 * gn + 2 * inner + h] = expf(-expf(a_log[h]) * dt);
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < channels; c += SCAN_THREADS) {
+        float y = conv_b[c];
+        for (int j = 0; j < taps; ++j) {
+            const int at = t - (taps - 1) + j;      // the row of the input `taps - 1 - j` tokens back
+            const float in = at >= first ? proj[(size_t)at * stride + inner + c] : kept[(size_t)(taps - 1 + (at - first)) * channels + c];
+            y = fmaf(conv_w[(size_t)c * taps + j], in, y);
+        }
+        y = silu_f(y);
+        if (c < inner) {
+            dst[2 * gn + c] = dt_s[c / p] * y;
+            dst[2 * gn + inner + c] = y;
+        } else if (c < inner + gn) {
+            dst[gn + (c - inner)] = y;          // B: the keys
+        } else {
+            dst[c - inner - gn] = y;            // C: the queries
+        }
+    }
+}
+
+extern "C" int kipp_ssd_prepare(const float* proj, int stride, const float* conv_w, const float* conv_b, int taps, const float* a_log,
+                                const float* dt_bias, float* state, size_t state_stride, size_t kept_at, const int32_t* seq_of_token,
+                                const int32_t* q_start, const int32_t* q_len, const int32_t* slots, float* prep, int prep_stride,
+                                int tokens, int entries, int heads, int groups, int n, int p, hipStream_t stream) {
+    if (tokens <= 0) return 0;
+    if (taps < 1 || taps > MAX_TAPS || heads <= 0 || heads > SSD_MAX_HEADS || groups <= 0 || heads % groups || n <= 0 || p <= 0) return -1;
+    const int inner = heads * p, channels = inner + 2 * groups * n;
+    if (stride < inner + channels + heads || prep_stride < 2 * groups * n + 2 * inner + heads ||
+        state_stride < kept_at + (size_t)(taps - 1) * channels) return -1;
+    hipLaunchKernelGGL(ssd_prepare_kernel, dim3(tokens), dim3(SCAN_THREADS), 0, stream, proj, stride, conv_w, conv_b, taps, a_log, dt_bias,
+                       (const float*)state, state_stride, kept_at, seq_of_token, q_start, slots, prep, prep_stride, heads, groups, n, p);
+    if (taps > 1)
+        hipLaunchKernelGGL(conv_keep_kernel, dim3((channels + 255) / 256, entries), dim3(256), 0, stream, proj + inner, stride, taps, state,
+                           state_stride, kept_at, q_start, q_len, slots, channels);
+    return KIPP_LAUNCH_CHECK();
+}
+
+// y[t][c] = (o[t][c] + skip[c / p] x[t][c]) * silu(z[t][c]); out = y * rsqrt(mean over c's span of y^2 + eps) * w[c]: the gate
+// comes before the norm.  x at column `x_at` of prep, z at column `z_at` of proj.
+template <typename TO>
+__global__ void __launch_bounds__(SCAN_THREADS)
+ssd_finish_kernel(const float* __restrict__ o_raw, const float* __restrict__ prep, int prep_stride, int x_at,
+                  const float* __restrict__ proj, int proj_stride, int z_at, const float* __restrict__ skip, int p,
+                  const float* __restrict__ w, float eps, TO* __restrict__ out, int width, int span) {
+    __shared__ float scratch[16];
+    const size_t t = blockIdx.y;
+    const int c0 = blockIdx.x * span;
+    const float* o = o_raw + t * width + c0;
+    const float* x = prep + t * prep_stride + x_at + c0;
+    const float* z = proj + t * proj_stride + z_at + c0;
+    float ss = 0.0f;
+    for (int e = threadIdx.x; e < span; e += SCAN_THREADS) {
+        const float y = fmaf(skip[(c0 + e) / p], x[e], o[e]) * silu_f(z[e]);
+        ss = fmaf(y, y, ss);
+    }
+    const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)span + eps);
+    for (int e = threadIdx.x; e < span; e += SCAN_THREADS) {
+        const float y = fmaf(skip[(c0 + e) / p], x[e], o[e]) * silu_f(z[e]);
+        store_f(out, t * width + c0 + e, y * inv * w[c0 + e]);
+    }
+}
+
+extern "C" int kipp_ssd_finish(const float* o_raw, const float* prep, int prep_stride, int x_at, const float* proj, int proj_stride,
+                               int z_at, const float* skip, int p, const float* w, float eps, void* out, int out_dtype, int tokens,
+                               int width, int span, hipStream_t stream) {
+    if (tokens <= 0) return 0;
+    if (width <= 0 || span <= 0 || width % span || p <= 0 || width % p || prep_stride < x_at + width || proj_stride < z_at + width) return -1;
+    dim3 grid(width / span, tokens), block(SCAN_THREADS);
+    if (out_dtype == KIPP_F32)
+        hipLaunchKernelGGL((ssd_finish_kernel<float>), grid, block, 0, stream, o_raw, prep, prep_stride, x_at, proj, proj_stride, z_at, skip, p,
+                           w, eps, (float*)out, width, span);
+    else if (out_dtype == KIPP_BF16)
+        hipLaunchKernelGGL((ssd_finish_kernel<bf16_t>), grid, block, 0, stream, o_raw, prep, prep_stride, x_at, proj, proj_stride, z_at, skip, p,
+                           w, eps, (bf16_t*)out, width, span);
+    else
+        return -2;
     return KIPP_LAUNCH_CHECK();
 }
 

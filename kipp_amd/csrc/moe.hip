@@ -3,6 +3,9 @@
 //
 //     route    p = softmax(z) over all experts (float32); the `top` largest p (the lower index first among equals);
 //              weight = p / (sum of the chosen p + eps)
+//     route (grouped)  s = sigmoid(z); choice scores c = s + correction; experts in equal groups of neighbours, a group's
+//              score the sum of its two largest c; only experts of the `keep` best groups can be chosen; the `top` largest
+//              c among them; weight = s / (sum of the chosen s + eps) * scale
 //     sort     the (token, choice) pairs in runs of one expert each, cut into tiles of up to 16 (or 128) rows; the list of tiles
 //              is made on the device, so the host never learns the counts and the launches have a fixed shape
 //     expert   a tile's rows against its expert's matrix: out[row][n] = act(sum_k W_e[n][k] x[row][k]).  bfloat16 with K a
@@ -29,7 +32,7 @@
 #define MFMA_THREADS 256
 #define XCDS 8              // dies of the chip; consecutive workgroups of a launch go to them in turn
 
-enum { ACT_NONE = -1, ACT_SILU = 0, ACT_RELU = 1, ACT_GELU = 2, ACT_GELU_TANH = 3 };
+enum { ACT_NONE = -1, ACT_SILU = 0, ACT_RELU = 1, ACT_GELU = 2, ACT_GELU_TANH = 3, ACT_RELU2 = 4 };
 
 __device__ __forceinline__ float activate(float z, int act) {
     switch (act) {
@@ -37,6 +40,7 @@ __device__ __forceinline__ float activate(float z, int act) {
         case ACT_RELU: return fmaxf(z, 0.0f);
         case ACT_GELU: return 0.5f * z * (1.0f + erff(z * 0.70710678118654752440f));
         case ACT_GELU_TANH: return 0.5f * z * (1.0f + tanhf(0.79788456080286535588f * (z + 0.044715f * z * z * z)));
+        case ACT_RELU2: { const float r = fmaxf(z, 0.0f); return r * r; }
         default: return z;
     }
 }
@@ -93,6 +97,92 @@ moe_route_kernel(const float* __restrict__ z, int parts, size_t part_stride, int
     if (lane < top) {
         chosen[(size_t)t * top + lane] = mine_e;
         weight[(size_t)t * top + lane] = mine / (picked_sum + eps);
+    }
+}
+
+// One wave a token: sigmoid scores, a correction for the choice alone, groups of neighbouring experts of which the best stay.
+__global__ void __launch_bounds__(ROUTE_WAVES * KIPP_WAVE)
+moe_route_grouped_kernel(const float* __restrict__ z, int parts, size_t part_stride, int stride, const float* __restrict__ correction,
+                         int32_t* __restrict__ chosen, float* __restrict__ weight, int tokens, int experts, int top, float eps,
+                         int group_count, int group_keep, float scale) {
+    __shared__ float c_s[ROUTE_WAVES][MAX_EXPERTS];     // choice scores, then -inf for experts of groups that do not stay
+    __shared__ float g_s[ROUTE_WAVES][MAX_EXPERTS];     // group scores, -inf once a group is taken
+    const int wave = threadIdx.x / KIPP_WAVE, lane = threadIdx.x & (KIPP_WAVE - 1);
+    int t = blockIdx.x * ROUTE_WAVES + wave;
+    const bool live = t < tokens;
+    if (!live) t = tokens - 1;      // stay in step with the barriers
+    const int size = experts / group_count;
+    float s[MAX_EXPERTS / KIPP_WAVE];
+#pragma unroll
+    for (int i = 0; i < MAX_EXPERTS / KIPP_WAVE; ++i) {
+        const int e = lane + i * KIPP_WAVE;
+        s[i] = 0.0f;
+        if (e < experts) {
+            float v = z[(size_t)t * stride + e];
+            for (int q = 1; q < parts; ++q) v += z[q * part_stride + (size_t)t * stride + e];
+            s[i] = 1.0f / (1.0f + expf(-v));
+            c_s[wave][e] = s[i] + (correction != nullptr ? correction[e] : 0.0f);
+        }
+    }
+    __syncthreads();
+    if (group_keep < group_count) {
+        for (int g = lane; g < group_count; g += KIPP_WAVE) {
+            float a = -INFINITY, b = -INFINITY;      // the two largest of the group
+            for (int j = 0; j < size; ++j) {
+                const float v = c_s[wave][g * size + j];
+                if (v > a) { b = a; a = v; } else if (v > b) { b = v; }
+            }
+            g_s[wave][g] = size > 1 ? a + b : a;
+        }
+        __syncthreads();
+        for (int round = 0; round < group_keep; ++round) {
+            float best = -INFINITY;
+            int best_g = MAX_EXPERTS;
+            for (int g = lane; g < group_count; g += KIPP_WAVE) {
+                const float v = g_s[wave][g];
+                if (v > best || (best_g == MAX_EXPERTS && v != -INFINITY)) { best = v; best_g = g; }
+            }
+            for (int off = 32; off > 0; off >>= 1) {
+                const float ob = __shfl_xor(best, off, KIPP_WAVE);
+                const int og = __shfl_xor(best_g, off, KIPP_WAVE);
+                if (og != MAX_EXPERTS && (best_g == MAX_EXPERTS || ob > best || (ob == best && og < best_g))) { best = ob; best_g = og; }
+            }
+            __syncthreads();
+            if (lane == 0 && best_g != MAX_EXPERTS) g_s[wave][best_g] = -INFINITY;      // taken: it stays
+            __syncthreads();
+        }
+        for (int e = lane; e < experts; e += KIPP_WAVE)
+            if (g_s[wave][e / size] != -INFINITY) c_s[wave][e] = -INFINITY;             // its group was not taken
+        __syncthreads();
+    }
+    float c[MAX_EXPERTS / KIPP_WAVE];
+#pragma unroll
+    for (int i = 0; i < MAX_EXPERTS / KIPP_WAVE; ++i) {
+        const int e = lane + i * KIPP_WAVE;
+        c[i] = e < experts ? c_s[wave][e] : -INFINITY;
+    }
+    float picked_sum = 0.0f, mine = 0.0f;       // lane j keeps the j-th choice
+    int mine_e = 0;
+    for (int j = 0; j < top; ++j) {
+        float best = -INFINITY, best_s = 0.0f;
+        int best_e = MAX_EXPERTS;
+#pragma unroll
+        for (int i = 0; i < MAX_EXPERTS / KIPP_WAVE; ++i)
+            if (c[i] > best) { best = c[i]; best_e = lane + i * KIPP_WAVE; best_s = s[i]; }     // the lowest index of a lane's largest
+        for (int off = 32; off > 0; off >>= 1) {
+            const float ob = __shfl_xor(best, off, KIPP_WAVE), os = __shfl_xor(best_s, off, KIPP_WAVE);
+            const int oe = __shfl_xor(best_e, off, KIPP_WAVE);
+            if (ob > best || (ob == best && oe < best_e)) { best = ob; best_e = oe; best_s = os; }
+        }
+#pragma unroll
+        for (int i = 0; i < MAX_EXPERTS / KIPP_WAVE; ++i)
+            if (lane + i * KIPP_WAVE == best_e) c[i] = -INFINITY;
+        picked_sum += best_s;
+        if (lane == j) { mine = best_s; mine_e = best_e < experts ? best_e : 0; }
+    }
+    if (live && lane < top) {
+        chosen[(size_t)t * top + lane] = mine_e;
+        weight[(size_t)t * top + lane] = mine / (picked_sum + eps) * scale;
     }
 }
 
@@ -332,11 +422,31 @@ extern "C" int kipp_moe_route(const float* z, int parts, int stride, int32_t* ch
     return KIPP_LAUNCH_CHECK();
 }
 
+// The same with sigmoid scores, a correction of the choice (or none) and groups of which `group_keep` of `group_count` stay.
+extern "C" int kipp_moe_route_grouped(const float* z, int parts, int stride, const float* correction, int32_t* chosen, float* weight,
+                                      int tokens, int experts, int top, float eps, int group_count, int group_keep, float scale,
+                                      int32_t* pair_token, int32_t* place_of_pair, int32_t* tiles, int max_tiles, int tile_rows,
+                                      hipStream_t stream) {
+    if (tokens <= 0) return 0;
+    if (experts <= 0 || experts > MAX_EXPERTS || top <= 0 || top > MAX_TOP || top > experts || stride < experts || parts <= 0) return -1;
+    if (group_count <= 0 || experts % group_count || group_keep <= 0 || group_keep > group_count ||
+        top > group_keep * (experts / group_count)) return -1;
+    const int pairs = tokens * top;
+    if (tile_rows != TILE_ROWS && tile_rows != MFMA_ROWS) return -1;
+    if (max_tiles < (pairs + tile_rows - 1) / tile_rows + (experts < pairs ? experts : pairs)) return -1;
+    hipLaunchKernelGGL(moe_route_grouped_kernel, dim3((tokens + ROUTE_WAVES - 1) / ROUTE_WAVES), dim3(ROUTE_WAVES * KIPP_WAVE), 0, stream, z,
+                       parts, (size_t)tokens * stride, stride, correction, chosen, weight, tokens, experts, top, eps, group_count, group_keep,
+                       scale);
+    hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, stream, (const int32_t*)chosen, pairs, experts, top, pair_token,
+                       place_of_pair, tiles, max_tiles, tile_rows);
+    return KIPP_LAUNCH_CHECK();
+}
+
 // `tile_rows`: the rows of the tiles that `kipp_moe_route` was asked for: 128 takes the matrix cores (bfloat16 x and w, K a multiple of 32), 16 the plain kernel.
 extern "C" int kipp_moe_expert(const void* x, int x_dtype, const int32_t* gather, const void* w, int w_dtype, const int32_t* tiles,
                                int max_tiles, void* out, int out_dtype, int n_out, int k, int act, int tile_rows, hipStream_t stream) {
     if (max_tiles <= 0) return 0;
-    if (n_out <= 0 || k <= 0 || act < ACT_NONE || act > ACT_GELU_TANH) return -1;
+    if (n_out <= 0 || k <= 0 || act < ACT_NONE || act > ACT_RELU2) return -1;
     if (tile_rows == MFMA_ROWS) {
         if (x_dtype != KIPP_BF16 || w_dtype != KIPP_BF16 || k % 32) return -2;
         // a lane's offsets into x and into an expert's matrix are 32 bits wide
@@ -374,10 +484,11 @@ extern "C" int kipp_moe_combine(const float* y, const int32_t* place, const floa
     return KIPP_LAUNCH_CHECK();
 }
 
-// out[r][i] = act(sum of the slabs of u[r][i]) [* sum of the slabs of u[r][inner + i] when `glu`]
+// out[r][i] = act(sum of the slabs of u[r][i]) [* sum of the slabs of u[r][inner + i] when `glu`]; with `bias` (over u's
+// columns) each sum has its column's bias added first
 template <typename TO>
 __global__ void activate_kernel(const float* __restrict__ u, int parts, size_t part_stride, TO* __restrict__ out, size_t total,
-                                int inner, int glu, int act) {
+                                int inner, int glu, int act, const float* __restrict__ bias) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= total) return;
     const size_t r = i / inner;
@@ -388,21 +499,30 @@ __global__ void activate_kernel(const float* __restrict__ u, int parts, size_t p
         a += u[p * part_stride + at];
         if (glu) b += u[p * part_stride + at + inner];
     }
+    if (bias != nullptr) {
+        a += bias[c];
+        if (glu) b += bias[inner + c];
+    }
     store_f(out, i, glu ? activate(a, act) * b : activate(a, act));
 }
 
-extern "C" int kipp_activate(const float* u, int parts, void* out, int out_dtype, int rows, int inner, int glu, int act,
-                             hipStream_t stream) {
+extern "C" int kipp_activate_biased(const float* u, int parts, void* out, int out_dtype, int rows, int inner, int glu, int act,
+                                    const float* bias, hipStream_t stream) {
     if (rows <= 0) return 0;
-    if (inner <= 0 || parts <= 0 || act < ACT_SILU || act > ACT_GELU_TANH) return -1;
+    if (inner <= 0 || parts <= 0 || act < ACT_SILU || act > ACT_RELU2) return -1;
     const size_t total = (size_t)rows * inner;
     const size_t part_stride = total * (glu ? 2 : 1);
     dim3 grid((unsigned)((total + 255) / 256)), block(256);
     if (out_dtype == KIPP_F32)
-        hipLaunchKernelGGL((activate_kernel<float>), grid, block, 0, stream, u, parts, part_stride, (float*)out, total, inner, glu, act);
+        hipLaunchKernelGGL((activate_kernel<float>), grid, block, 0, stream, u, parts, part_stride, (float*)out, total, inner, glu, act, bias);
     else if (out_dtype == KIPP_BF16)
-        hipLaunchKernelGGL((activate_kernel<bf16_t>), grid, block, 0, stream, u, parts, part_stride, (bf16_t*)out, total, inner, glu, act);
+        hipLaunchKernelGGL((activate_kernel<bf16_t>), grid, block, 0, stream, u, parts, part_stride, (bf16_t*)out, total, inner, glu, act, bias);
     else
         return -2;
     return KIPP_LAUNCH_CHECK();
+}
+
+extern "C" int kipp_activate(const float* u, int parts, void* out, int out_dtype, int rows, int inner, int glu, int act,
+                             hipStream_t stream) {
+    return kipp_activate_biased(u, parts, out, out_dtype, rows, inner, glu, act, nullptr, stream);
 }

@@ -157,6 +157,18 @@ def residual_add(x: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
     return x
 
 
+def residual_add_scaled(x: torch.Tensor, delta: torch.Tensor, scale: float = 1.0, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x += scale * (delta + bias): `delta` float32 of x's shape or slabs of it (added in order), `bias` float32 [width] or none."""
+    _dev(x, delta, bias)
+    _need(x.dtype == delta.dtype == torch.float32 and x.dim() == 2 and tuple(delta.shape[-2:]) == tuple(x.shape) and delta.dim() in (2, 3),
+          "residual_add_scaled: float32 x [rows, width] and a float32 delta of its shape (or slabs of it)")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == x.shape[1]), "residual_add_scaled: float32 bias [width]")
+    parts = delta.shape[0] if delta.dim() == 3 else 1
+    fn = _fn("elementwise", "kipp_residual_add_scaled", [_c_ptr, _c_ptr, _c_int, _c_size, _c_float, _c_ptr, _c_int, _c_ptr])
+    _check(fn(_ptr(x), _ptr(delta), parts, x.numel(), float(scale), _ptr(bias), x.shape[1], _stream()), "residual_add_scaled")
+    return x
+
+
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor, pairs: bool = False) -> torch.Tensor:
     """out[t, i] = silu(gate_up[t, i]) * gate_up[t, inner + i]; `gate_up` is
     [rows, 2 inner] or slabs [parts, rows, 2 inner] that are added in order.
@@ -400,14 +412,29 @@ def head_prepare(proj: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor,
                  n_q: int, n_kv: int, d: int, dv: int, bias: Optional[torch.Tensor], norm: str, eps: float,
                  q_norm_w: Optional[torch.Tensor] = None, k_norm_w: Optional[torch.Tensor] = None,
                  temp_coef: float = 0.0, temp_every: int = 0, write_kv: bool = True,
-                 q_head_scale: Optional[torch.Tensor] = None, v_norm_eps: Optional[float] = None) -> torch.Tensor:
+                 q_head_scale: Optional[torch.Tensor] = None, v_norm_eps: Optional[float] = None,
+                 angles: Optional[torch.Tensor] = None, rotary_dim: int = 0, v_first_in: Optional[torch.Tensor] = None,
+                 v_first_out: Optional[torch.Tensor] = None, v_lambda: Optional[torch.Tensor] = None) -> torch.Tensor:
     """From a step's input product `proj` (float32 [tokens, >= n_q d + n_kv d + n_kv dv], columns q | k | v | ..., or slabs
     of it): `bias` added (float32 over the q | k | v columns), every head of q and k RMS-normed (`norm`: "none", "plain"
     or "weighted" with `q_norm_w` / `k_norm_w` [d]), queries at position p times 1 + temp_coef ln(floor((p + 1) /
     temp_every) + 1) (temp_every 0: none), queries of head h times `q_head_scale[h]` (float32 [n_q]), every value head over
     its root mean square with `v_norm_eps` inside the root (None: values as they are), q kept in `q_out`, k and v written
-    into the pages of their positions."""
-    _dev(proj, q_out, k_cache, v_cache, positions, seq_of_token, block_table, bias, q_norm_w, k_norm_w, q_head_scale)
+    into the pages of their positions.  `angles` (`rotary_angles`, float32 [tokens, rotary_dim]): after the norm the first
+    `rotary_dim` numbers of every q and k head are turned, number i with number i + rotary_dim / 2.  `v_first_out` (float32
+    [tokens, n_kv dv]) receives the values as they are; with `v_first_in` (another layer's, of the same tokens) and `v_lambda`
+    (float32, one number on the device) the value that is cached is (1 - lambda) v + lambda v_first."""
+    _dev(proj, q_out, k_cache, v_cache, positions, seq_of_token, block_table, bias, q_norm_w, k_norm_w, q_head_scale, angles,
+         v_first_in, v_first_out, v_lambda)
+    if angles is not None:
+        _need(0 < rotary_dim <= d and rotary_dim % 2 == 0, "head_prepare: rotary_dim is even and at most d")
+        _angles_ok(angles, proj.shape[-2], rotary_dim, "head_prepare")
+    for vf in (v_first_in, v_first_out):
+        if vf is not None:
+            _need(write_kv and vf.dtype == torch.float32 and tuple(vf.shape) == (proj.shape[-2], n_kv * dv), "head_prepare: first values are float32 [tokens, n_kv dv]")
+    if v_first_in is not None:
+        _need(v_lambda is not None and v_lambda.dtype == torch.float32 and v_lambda.numel() == 1 and v_first_in is not v_first_out,
+              "head_prepare: mixing values needs a float32 lambda on the device")
     if q_head_scale is not None:
         _need(q_head_scale.dtype == torch.float32 and q_head_scale.numel() == n_q, "head_prepare: float32 q_head_scale [n_q]")
     _need(v_norm_eps is None or v_norm_eps >= 0, "head_prepare: v_norm_eps must not be negative")
@@ -427,23 +454,27 @@ def head_prepare(proj: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor,
           and k_cache.shape[3] == d and v_cache.shape[3] == dv and k_cache.dtype == v_cache.dtype,
           "head_prepare: caches must be [pages, n_kv, page, d] and [pages, n_kv, page, dv]")
     _need(block_table.dim() == 2 and int(temp_every) >= 0, "head_prepare: block_table is [sequences, blocks]")
-    fn = _fn("head_prepare", "kipp_head_prepare_scaled",
+    fn = _fn("head_prepare", "kipp_head_prepare_rotated",
              [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
-              _c_int, _c_ptr, _c_ptr, _c_float, _c_float, _c_int] + [_c_int] * 7 + [_c_ptr, _c_float, _c_ptr])
+              _c_int, _c_ptr, _c_ptr, _c_float, _c_float, _c_int] + [_c_int] * 7 + [_c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr])
     _check(fn(_ptr(proj), parts, stride, _ptr(bias), _ptr(q_out), _code(q_out), _ptr(k_cache), _ptr(v_cache), _code(k_cache),
               _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1],
               {"none": 0, "plain": 1, "weighted": 2}[norm], _ptr(q_norm_w), _ptr(k_norm_w), float(eps), float(temp_coef),
               int(temp_every), n, n_q, n_kv, d, dv, k_cache.shape[2], int(write_kv), _ptr(q_head_scale),
-              -1.0 if v_norm_eps is None else float(v_norm_eps), _stream()), "head_prepare")
+              -1.0 if v_norm_eps is None else float(v_norm_eps), _ptr(angles), int(rotary_dim) if angles is not None else 0,
+              _ptr(v_first_in), _ptr(v_first_out), _ptr(v_lambda), _stream()), "head_prepare")
     return q_out
 
 
 def paged_attention_wide(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                          positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
-                         n_q: int, n_kv: int, d: int, dv: int, scale: float, window: int = 0, softcap: float = 0.0) -> torch.Tensor:
+                         n_q: int, n_kv: int, d: int, dv: int, scale: float, window: int = 0, softcap: float = 0.0,
+                         chunk: int = 0, sink: bool = False) -> torch.Tensor:
     """The generic attention kernel with values of their own width: keys of up to 1,024 numbers, values of `dv`.
     `v_cache` may be `k_cache` itself: a value is then the first dv numbers of its key's row.  `softcap` c > 0: a
-    scaled score s becomes c tanh(s / c)."""
+    scaled score s becomes c tanh(s / c).  `chunk` c > 0 (instead of a window): position p sees the keys from p - p % c
+    on.  `sink`: one is added to the softmax's denominator (a key of score 0 that has no value)."""
+    _need(chunk >= 0 and not (chunk and window), "attention: a chunk or a window, not both")
     _dev(q, k_cache, v_cache, out, positions, seq_of_token, block_table)
     for t, name in ((positions, "positions"), (seq_of_token, "seq_of_token"), (block_table, "block_table")):
         _i32(t, name)
@@ -455,12 +486,13 @@ def paged_attention_wide(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.
     _need(positions.numel() == n and seq_of_token.numel() == n and block_table.dim() == 2,
           "attention: one position and sequence per token, block_table [sequences, blocks]")
     _need(softcap >= 0, "attention: softcap must not be negative")
-    fn = _fn("attention_generic", "kipp_paged_attention_generic_capped",
+    fn = _fn("attention_generic", "kipp_paged_attention_generic_masked",
              [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
-              _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_float, _c_ptr])
+              _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_float, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(q), _code(q), _ptr(k_cache), _ptr(v_cache), _code(k_cache), _ptr(out), _code(out),
               _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1],
-              n, n_q, n_kv, d, dv, v_cache.shape[3], k_cache.shape[2], float(scale), int(window), float(softcap), _stream()),
+              n, n_q, n_kv, d, dv, v_cache.shape[3], k_cache.shape[2], float(scale), int(window), float(softcap), int(chunk),
+              int(bool(sink)), _stream()),
            "paged_attention_wide")
     return out
 
@@ -700,6 +732,80 @@ def delta_scan(prep: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor, q
     return o_raw
 
 
+def ssd_state_size(heads: int, groups: int, n: int, p: int, taps: int) -> int:
+    """float32 numbers of a request's state: S [heads, p, n], then the last taps - 1 inputs of the x | B | C channels."""
+    size = heads * n * p + (taps - 1) * (heads * p + 2 * groups * n)
+    return -(-size // 4) * 4
+
+
+def ssd_prep_width(heads: int, groups: int, n: int, p: int) -> int:
+    """Columns of what `ssd_prepare` writes: C | B | dt x | x | g."""
+    return 2 * groups * n + 2 * heads * p + heads
+
+
+def ssd_prepare(proj: torch.Tensor, conv_w: torch.Tensor, conv_b: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
+                state: torch.Tensor, seq_of_token: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor, slots: torch.Tensor,
+                prep: torch.Tensor, heads: int, groups: int, n: int, p: int) -> torch.Tensor:
+    """The state space recurrence's inputs from its input product `proj` (float32 [tokens, z | x | B | C | dt], z and x of
+    heads p columns, B and C of groups n, dt of heads): x, B and C behind their short causal filter (`conv_w` [channels,
+    taps], `conv_b` [channels], the slot's kept inputs ahead of a portion) and silu; dt = softplus(dt + dt_bias);
+    `prep` [tokens, `ssd_prep_width`] receives C | B | dt x | x | g with g = exp(-exp(a_log) dt) a head.  The slot's kept
+    inputs are then moved on by the portion."""
+    _dev(proj, conv_w, conv_b, a_log, dt_bias, state, seq_of_token, q_start, q_len, slots, prep)
+    for t, name in ((seq_of_token, "seq_of_token"), (q_start, "q_start"), (q_len, "q_len"), (slots, "slots")):
+        _i32(t, name)
+    inner, channels = heads * p, heads * p + 2 * groups * n
+    tokens = proj.shape[0]
+    _need(proj.dim() == 2 and proj.dtype == torch.float32 and proj.shape[1] >= inner + channels + heads, "ssd_prepare: proj is float32 [tokens, z | x | B | C | dt]")
+    _need(conv_w.dtype == conv_b.dtype == torch.float32 and conv_w.dim() == 2 and conv_w.shape[0] == channels and conv_b.numel() == channels
+          and 1 <= conv_w.shape[1] <= 16, "ssd_prepare: float32 filters [channels, taps] with a bias a channel, up to 16 taps")
+    taps = conv_w.shape[1]
+    _need(a_log.dtype == dt_bias.dtype == torch.float32 and a_log.numel() == dt_bias.numel() == heads and 0 < heads <= 1024 and heads % groups == 0,
+          "ssd_prepare: float32 a_log and dt_bias [heads], up to 1,024 heads in equal groups")
+    _need(prep.dtype == torch.float32 and prep.shape == (tokens, ssd_prep_width(heads, groups, n, p)) and seq_of_token.numel() == tokens,
+          "ssd_prepare: prep is float32 [tokens, 2 groups n + 2 heads p + heads]")
+    _need(state.dim() == 2 and state.dtype == torch.float32 and state.shape[1] >= ssd_state_size(heads, groups, n, p, taps), "ssd_prepare: state is float32 [slots, size]")
+    _need(q_start.numel() == q_len.numel() == slots.numel(), "ssd_prepare: one start, length and slot an entry")
+    fn = _fn("linear_scan", "kipp_ssd_prepare", [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_size, _c_size, _c_ptr, _c_ptr, _c_ptr,
+                                                 _c_ptr, _c_ptr, _c_int] + [_c_int] * 6 + [_c_ptr])
+    _check(fn(_ptr(proj), proj.shape[1], _ptr(conv_w), _ptr(conv_b), taps, _ptr(a_log), _ptr(dt_bias), _ptr(state), state.shape[1], heads * n * p,
+              _ptr(seq_of_token), _ptr(q_start), _ptr(q_len), _ptr(slots), _ptr(prep), prep.shape[1], tokens, q_start.numel(), heads, groups, n, p,
+              _stream()), "ssd_prepare")
+    return prep
+
+
+def gated_scan(prep: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor, slots: torch.Tensor,
+               o_raw: torch.Tensor, heads: int, groups: int, n: int, p: int, longest: int = 0) -> torch.Tensor:
+    """The recurrence with a decay a token and head over every entry's tokens, in order, from and into the entry's slot:
+    S <- g S + k v^T; o = S^T q, with `prep` as `ssd_prepare` leaves it (q = C, k = B shared by the heads of a group, v = dt x).
+    `longest` as for `decay_scan`."""
+    _dev(prep, state, q_start, q_len, slots, o_raw)
+    _need(prep.dim() == 2 and prep.dtype == torch.float32 and prep.shape[1] >= ssd_prep_width(heads, groups, n, p) and heads % groups == 0,
+          "gated_scan: prep is float32 [tokens, C | B | dt x | x | g]")
+    _scan_args(state, q_start, q_len, slots, o_raw, prep.shape[0], heads, n, p, "gated_scan")
+    fn = _fn("linear_scan", "kipp_gated_scan", [_c_ptr, _c_int, _c_ptr, _c_size, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(prep), prep.shape[1], _ptr(state), state.shape[1], _ptr(q_start), _ptr(q_len), _ptr(slots), _ptr(o_raw), q_start.numel(),
+              heads, groups, n, p, max(0, int(longest)), _stream()), "gated_scan")
+    return o_raw
+
+
+def ssd_finish(o_raw: torch.Tensor, prep: torch.Tensor, x_at: int, proj: torch.Tensor, z_at: int, skip: torch.Tensor, p: int,
+               norm_w: torch.Tensor, eps: float, span: int, out: torch.Tensor) -> torch.Tensor:
+    """out [tokens, width]: y = (o_raw + skip[column // p] x) silu(z), x at column `x_at` of `prep` and z at column `z_at` of
+    `proj`; then every run of `span` columns of y over its root mean square, times norm_w[column] (the gate before the norm)."""
+    _dev(o_raw, prep, proj, skip, norm_w, out)
+    tokens, width = o_raw.shape
+    _need(o_raw.dtype == prep.dtype == proj.dtype == skip.dtype == norm_w.dtype == torch.float32 and out.shape == o_raw.shape
+          and prep.dim() == proj.dim() == 2 and prep.shape[0] == proj.shape[0] == tokens and prep.shape[1] >= x_at + width
+          and proj.shape[1] >= z_at + width and width % span == 0 and width % p == 0 and skip.numel() == width // p and norm_w.numel() == width,
+          "ssd_finish: float32 rows, x and z columns inside their rows, one skip a head, a weight a column")
+    fn = _fn("linear_scan", "kipp_ssd_finish", [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_ptr, _c_float, _c_ptr, _c_int,
+                                                _c_int, _c_int, _c_int, _c_ptr])
+    _check(fn(_ptr(o_raw), _ptr(prep), prep.shape[1], int(x_at), _ptr(proj), proj.shape[1], int(z_at), _ptr(skip), int(p), _ptr(norm_w), float(eps),
+              _ptr(out), _code(out), tokens, width, int(span), _stream()), "ssd_finish")
+    return out
+
+
 def scan_finish(o_raw: torch.Tensor, gates: torch.Tensor, gate_at: int, norm_w: torch.Tensor, eps: float, gate: str, span: int,
                 out: torch.Tensor) -> torch.Tensor:
     """out [tokens, width] = every run of `span` columns of `o_raw` over its root mean square, times norm_w[column % len(norm_w)],
@@ -716,7 +822,7 @@ def scan_finish(o_raw: torch.Tensor, gates: torch.Tensor, gate_at: int, norm_w: 
 
 # --------------------------------------------------------------------------- routed feed-forward
 
-ACTIVATIONS = {"silu": 0, "relu": 1, "gelu": 2, "gelu_tanh": 3}
+ACTIVATIONS = {"silu": 0, "relu": 1, "gelu": 2, "gelu_tanh": 3, "relu2": 4}     # relu2: the square of relu
 MOE_TILE_ROWS = 16
 MOE_MFMA_ROWS = 128    # rows of a tile of the experts' products on the matrix cores
 
@@ -734,7 +840,8 @@ def moe_max_tiles(tokens: int, experts: int, top: int, tile_rows: int = 16) -> i
 
 
 def moe_route(z: torch.Tensor, experts: int, top: int, eps: float, chosen: torch.Tensor, weight: torch.Tensor,
-              pair_token: torch.Tensor, place_of_pair: torch.Tensor, tiles: torch.Tensor, tile_rows: int = 16):
+              pair_token: torch.Tensor, place_of_pair: torch.Tensor, tiles: torch.Tensor, tile_rows: int = 16,
+              router: str = "softmax", correction: Optional[torch.Tensor] = None, groups: Optional[tuple] = None, scale: float = 1.0):
     """From router logits `z` (float32 [tokens, >= experts] or slabs): softmax over the experts, the `top` largest a token
     (`chosen`, int32 [tokens, top]) with weights p / (sum of the chosen p + eps) (`weight`, float32 [tokens, top]); then the
     pairs sorted by expert: `pair_token` [pairs] the token of every sorted row, `place_of_pair` [pairs] the row of pair
@@ -747,6 +854,19 @@ def moe_route(z: torch.Tensor, experts: int, top: int, eps: float, chosen: torch
     _need(chosen.shape == (n, top) and weight.shape == (n, top) and weight.dtype == torch.float32 and pair_token.numel() == n * top
           and place_of_pair.numel() == n * top and tiles.dim() == 2 and tiles.shape[1] == 3 and tiles.shape[0] >= moe_max_tiles(n, experts, top, tile_rows),
           "moe_route: output shapes")
+    _need(router in ("softmax", "sigmoid"), "moe_route: router is softmax or sigmoid")
+    if router == "sigmoid":
+        _dev(correction)
+        count, keep = groups if groups is not None else (1, 1)
+        _need(correction is None or (correction.dtype == torch.float32 and correction.numel() == experts), "moe_route: float32 correction [experts]")
+        _need(count > 0 and experts % count == 0 and 0 < keep <= count and top <= keep * (experts // count),
+              "moe_route: equal groups, of which at least one stays, with experts enough for a token's choice")
+        fn = _fn("moe", "kipp_moe_route_grouped", [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_float,
+                                                   _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr])
+        _check(fn(_ptr(z), parts, stride, _ptr(correction), _ptr(chosen), _ptr(weight), n, experts, top, float(eps), int(count), int(keep), float(scale),
+                  _ptr(pair_token), _ptr(place_of_pair), _ptr(tiles), tiles.shape[0], int(tile_rows), _stream()), "moe_route")
+        return chosen, weight
+    _need(correction is None and groups is None and scale == 1.0, "moe_route: correction, groups and scale belong to the sigmoid router")
     fn = _fn("moe", "kipp_moe_route", [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr])
     _check(fn(_ptr(z), parts, stride, _ptr(chosen), _ptr(weight), n, experts, top, float(eps), _ptr(pair_token), _ptr(place_of_pair), _ptr(tiles),
               tiles.shape[0], int(tile_rows), _stream()), "moe_route")
@@ -790,14 +910,16 @@ def moe_combine(y: torch.Tensor, place_of_pair: torch.Tensor, weight: torch.Tens
     return out
 
 
-def activate(u: torch.Tensor, out: torch.Tensor, activation: str, glu: bool = False) -> torch.Tensor:
-    """out = act(u), or with `glu` out[r, i] = act(u[r, i]) * u[r, inner + i]; `u` float32 [rows, width] or slabs of it."""
-    _dev(u, out)
+def activate(u: torch.Tensor, out: torch.Tensor, activation: str, glu: bool = False, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = act(u), or with `glu` out[r, i] = act(u[r, i]) * u[r, inner + i]; `u` float32 [rows, width] or slabs of it;
+    `bias` (float32 [width]) is added to u's columns first."""
+    _dev(u, out, bias)
     parts, rows, width = _slabs(u, "activate")
     inner = out.shape[1]
     _need(out.shape[0] == rows and width == (2 * inner if glu else inner) and activation in ACTIVATIONS, "activate: shapes or activation")
-    fn = _fn("moe", "kipp_activate", [_c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
-    _check(fn(_ptr(u), parts, _ptr(out), _code(out), rows, inner, int(glu), ACTIVATIONS[activation], _stream()), "activate")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == width), "activate: float32 bias over u's columns")
+    fn = _fn("moe", "kipp_activate_biased", [_c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr])
+    _check(fn(_ptr(u), parts, _ptr(out), _code(out), rows, inner, int(glu), ACTIVATIONS[activation], _ptr(bias), _stream()), "activate")
     return out
 
 

@@ -34,6 +34,8 @@ def model_variants(spec, dtype: str) -> List[Spec]:
     owners = [("embedding", spec.embedding), ("norm", spec.final_norm), ("head", spec.head)]
     if getattr(spec, "input_position", None) is not None:
         owners.append(("position", spec.input_position))
+    if getattr(spec, "embedding_norm", None) is not None:
+        owners.append(("norm", spec.embedding_norm))
     for layer in spec.layers:
         block = part_class("block", layer.block)
         _add(out, getattr(block, "variants", lambda s, d: [])(layer, dtype))

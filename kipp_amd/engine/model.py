@@ -15,6 +15,8 @@ from ..weights.loader import check_tensors, read_model_tensors
 def _part_specs(spec: ModelSpec):
     """(category, part spec) of every part that owns tensors, in file order."""
     yield "embedding", spec.embedding
+    if spec.embedding_norm is not None:
+        yield "norm", spec.embedding_norm
     if spec.input_position is not None:
         yield "position", spec.input_position
     for layer in spec.layers:
@@ -54,6 +56,7 @@ class Model:
         self.spec = spec
         self.rt = runtime
         self.embedding = build_part("embedding", spec.embedding, runtime)
+        self.embedding_norm = build_part("norm", spec.embedding_norm, runtime) if spec.embedding_norm is not None else None
         self.input_position = (build_part("position", spec.input_position, runtime)
                                if spec.input_position is not None else None)
         self.blocks = [build_part("block", layer, runtime) for layer in spec.layers]
@@ -73,6 +76,8 @@ class Model:
     # -- weights ------------------------------------------------------------------------
     def _owners(self):
         yield "embedding", self.spec.embedding, self.embedding
+        if self.embedding_norm is not None:
+            yield "norm", self.spec.embedding_norm, self.embedding_norm
         if self.input_position is not None:
             yield "position", self.spec.input_position, self.input_position
         for layer, block in zip(self.spec.layers, self.blocks):
@@ -113,6 +118,8 @@ class Model:
         if self.spec.streams is not None:
             return self._forward_streams(batch, cache)
         x = self.embedding.forward(batch.tokens)
+        if self.embedding_norm is not None:
+            x = self.embedding_norm.forward(x, torch.float32)       # the residual stream starts as the normed rows
         if self.input_position is not None:
             x = self.input_position.forward(x, batch)
         pending = None

@@ -134,3 +134,40 @@ class SandwichNormMixerBlock(SandwichNormBlock):
     """The first half of the sandwich arrangement alone: a layer without a feed-forward."""
 
     roles = (("mixer_norm", "norm"), ("mixer", "mixer"), ("mixer_post_norm", "norm"))
+
+
+@register("block", "parallel")
+class ParallelBlock:
+    """One norm whose output both sublayers read: h = mixer_norm(x); x += mixer(h) + ffn(h).  The mixer's result is added
+    at once (a weighted sum of deltas term by term, where it lies); the feed-forward's is handed on and added inside the next
+    block's norm."""
+
+    roles = (("mixer_norm", "norm"), ("mixer", "mixer"), ("ffn", "feed_forward"))
+
+    def __init__(self, layer_spec, runtime):
+        self.rt = runtime
+        self.parts = {role: build_part(cat, layer_spec.part(role), runtime) for role, cat in self.roles}
+        self.mixer = self.parts["mixer"]
+        self.graph_safe = all(getattr(part, "graph_safe", False) for part in self.parts.values())
+
+    def forward(self, x, pending, batch, cache, state):
+        rt, norm = self.rt, self.parts["mixer_norm"]
+        if pending is not None and not getattr(norm, "fuses_products", False):
+            pending = rt.settle(pending)
+        h = norm.forward(x, rt.act_dtype) if pending is None else norm.add_forward(x, pending, rt.act_dtype)
+        h = rt.rows_of(h)       # two readers: the rows are finished once
+        delta = self.mixer.forward(h, batch, cache, state)
+        if hasattr(delta, "add_to"):
+            delta.add_to(x)
+        else:
+            rt.ops.residual_add(x, rt.settle(delta))
+        if "ffn" not in self.parts:
+            return x, None
+        return x, self.parts["ffn"].forward(h, batch)
+
+
+@register("block", "parallel_mixer")
+class ParallelMixerBlock(ParallelBlock):
+    """The parallel arrangement without a feed-forward."""
+
+    roles = (("mixer_norm", "norm"), ("mixer", "mixer"))

@@ -12,13 +12,14 @@ from __future__ import annotations
 
 import torch
 
-from ..runtime import ScaledRows, Weight
+from ..runtime import ScaledRows, Weight, WeightedDelta
 from .base import ParamSpec, register
 
 
 @register("feed_forward", "gated_mlp")
 class GatedMLP:
-    """delta = W_down (silu(W_gate x) * (W_up x))  (/root/reference/src/kipp.c:2633-2653)."""
+    """delta = W_down (silu(W_gate x) * (W_up x))  (/root/reference/src/kipp.c:2633-2653); with `bias_names` every
+    projection has a bias: the gate's and the up's are added in the activation's kernel, the down's rides on the delta."""
 
     graph_safe = True   # forward launches kernels only: no host reads, no data-dependent launches
     takes_scaled_rows = True
@@ -31,25 +32,42 @@ class GatedMLP:
     @staticmethod
     def params(spec):
         gate, up, down = spec.names
-        return {
+        p = {
             gate: ParamSpec((spec.intermediate_size, spec.hidden_size)),
             up: ParamSpec((spec.intermediate_size, spec.hidden_size)),
             down: ParamSpec((spec.hidden_size, spec.intermediate_size)),
         }
+        if getattr(spec, "bias_names", None) is not None:
+            for name, width in zip(spec.bias_names, (spec.intermediate_size, spec.intermediate_size, spec.hidden_size)):
+                p[name] = ParamSpec((width,), "float", ("normal", 0.1))
+        return p
+
+    @staticmethod
+    def placement(spec):
+        return {name: "float32" for name in (getattr(spec, "bias_names", None) or ())}
 
     def load(self, tensors):
         gate, up, down = self.spec.names
         g, u = tensors[gate], tensors[up]
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
-        self.w_gate_up = self.rt.weight(torch.cat([g, u], dim=0).contiguous(), gate_up=self.spec.activation == "silu")
+        biased = getattr(self.spec, "bias_names", None) is not None
+        self.w_gate_up = self.rt.weight(torch.cat([g, u], dim=0).contiguous(), gate_up=self.spec.activation == "silu" and not biased)
         self.w_down = self.rt.weight(tensors[down])
+        self.bias_gate_up = self.bias_down = None
+        if biased:
+            self.bias_gate_up = torch.cat([tensors[self.spec.bias_names[0]], tensors[self.spec.bias_names[1]]]).contiguous()
+            self.bias_down = tensors[self.spec.bias_names[2]]
 
     def forward(self, x, batch=None):
         rt = self.rt
         rows, inner = x.shape[0], self.spec.intermediate_size
         act = rt.empty((rows, inner), rt.act_dtype)
         w = self.w_gate_up
+        if self.bias_gate_up is not None:
+            # biases: the gate-up product by itself, then the activation's kernel adds them ahead of the activation
+            rt.ops.activate(rt.linear(rt.rows_of(x), w, slabs=True), act, self.spec.activation, glu=True, bias=self.bias_gate_up)
+            return WeightedDelta.of(rt, rt.linear(act, self.w_down, slabs=True, defer=True), 1.0, self.bias_down)
         if self.spec.activation != "silu":
             # another activation: the gate-up product by itself, then the activation's own kernel (the products that
             # end in the activation are built for silu)
@@ -98,6 +116,8 @@ class RoutedMLP:
         s = spec
         up, down = s.names
         p = {s.router_name: ParamSpec((s.experts, s.hidden_size))}
+        if getattr(s, "correction_name", None) is not None:
+            p[s.correction_name] = ParamSpec((s.experts,), "float", ("normal", 0.1))
         for e in range(s.experts):
             p[s.expert_prefix.format(e) + up] = ParamSpec((s.expert_size, s.hidden_size))
             p[s.expert_prefix.format(e) + down] = ParamSpec((s.hidden_size, s.expert_size))
@@ -107,12 +127,17 @@ class RoutedMLP:
         return p
 
     @staticmethod
+    def placement(spec):
+        return {spec.correction_name: "float32"} if getattr(spec, "correction_name", None) is not None else {}
+
+    @staticmethod
     def variants(spec, dtype):
         return [("moe", None)]
 
     def load(self, tensors):
         s = self.spec
         up, down = s.names
+        self.correction = tensors[s.correction_name] if getattr(s, "correction_name", None) is not None else None
         router = tensors[s.router_name]
         pad = -router.shape[0] % 16     # whole tiles of rows for the products
         if pad:
@@ -141,7 +166,11 @@ class RoutedMLP:
         # bfloat16 experts whose two contractions are multiples of 32 run on the matrix cores, in tiles of 128 rows
         tile_rows = ops.moe_tile_rows(self.w_up.dtype, s.hidden_size, s.expert_size)
         tiles = torch.empty((ops.moe_max_tiles(n, s.experts, s.top, tile_rows), 3), dtype=torch.int32, device=dev)
-        ops.moe_route(z, s.experts, s.top, s.weight_eps, chosen, weight, pair_token, place, tiles, tile_rows=tile_rows)
+        if s.router == "sigmoid":
+            ops.moe_route(z, s.experts, s.top, s.weight_eps, chosen, weight, pair_token, place, tiles, tile_rows=tile_rows, router="sigmoid",
+                          correction=self.correction, groups=s.groups, scale=s.route_scale)
+        else:
+            ops.moe_route(z, s.experts, s.top, s.weight_eps, chosen, weight, pair_token, place, tiles, tile_rows=tile_rows)
         if x.dtype != self.w_up.dtype:
             x = ops.cast(x, rt.empty(x.shape, self.w_up.dtype))
         inner = ops.moe_expert(x, pair_token, self.w_up, tiles, rt.empty((pairs, s.expert_size), self.w_up.dtype), s.activation, tile_rows=tile_rows)

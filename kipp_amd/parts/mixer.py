@@ -19,6 +19,8 @@ from __future__ import annotations
 
 import math
 
+import torch
+
 from ..cache.needs import KVNeed
 from .base import ParamSpec, build_part, register
 
@@ -57,12 +59,17 @@ class Attention:
             p[k_norm] = ParamSpec((spec.head_dim,), "float", ("one_plus_normal", 0.05))
         if spec.head_temp is not None:
             p[spec.head_temp] = ParamSpec((spec.num_heads,), "float", ("one_plus_normal", 0.2))
+        if spec.out_bias is not None:
+            p[spec.out_bias] = ParamSpec((spec.hidden_size,), "float", ("normal", 0.1))
+        if spec.v_mix is not None:
+            p[spec.v_mix_name] = ParamSpec((), "float", ("abs_normal", 0.3))
         return p
 
     @staticmethod
     def placement(spec):
         """What enters norms and sums in float32 is widened on the device (exact)."""
-        return {name: "float32" for name in spec.names[4:] + tuple(spec.bias_names) + ((spec.head_temp,) if spec.head_temp else ())}
+        return {name: "float32" for name in spec.names[4:] + tuple(spec.bias_names) + ((spec.head_temp,) if spec.head_temp else ())
+                + ((spec.out_bias,) if spec.out_bias else ()) + ((spec.v_mix_name,) if spec.v_mix else ())}
 
     @staticmethod
     def variants(spec, dtype):
@@ -70,7 +77,9 @@ class Attention:
         that share a key/value head).  Under float32, and for more than 16 heads a group, the generic
         attention kernel runs, which every model has."""
         out = [("rope_kv", None) if spec.plain else ("head_prepare", None), ("attention_generic", None)]
-        if dtype != "bfloat16" or spec.head_dim % 16 or spec.value_dim != spec.head_dim:
+        if not spec.plain and getattr(spec.position, "kind", "none") != "none":
+            out.append(("rope_kv", None))       # the step's table of angles
+        if dtype != "bfloat16" or spec.head_dim % 16 or spec.value_dim != spec.head_dim or spec.chunk is not None or spec.sink:
             return out
         group = spec.num_heads // spec.num_kv_heads
         capped = {"SOFTCAP": 1} if spec.softcap is not None else {}      # capped scores: builds of their own
@@ -104,12 +113,15 @@ class Attention:
             if not s.own_kv:        # the kernel's bias runs over q | k | v: nothing is added where nothing is written
                 held.append(torch.zeros(s.kv_dim + s.v_dim, dtype=torch.float32, device=held[0].device))
             self.bias = torch.cat([t.float() for t in held]).contiguous()
+        self.out_bias = tensors[s.out_bias] if s.out_bias is not None else None
+        self.v_lambda = tensors[s.v_mix_name].reshape(1).contiguous() if s.v_mix == "mix" else None
 
     @staticmethod
     def need_of(spec):
         """What a mixer of this spec keeps per token, known without building it."""
-        return KVNeed(num_kv_heads=spec.num_kv_heads, head_dim=spec.head_dim, window=spec.window, page_size=spec.page_size,
-                      v_head_dim=spec.v_head_dim)
+        # a chunk never reads further back than its own length: for the pages it is a window of that size
+        return KVNeed(num_kv_heads=spec.num_kv_heads, head_dim=spec.head_dim, window=spec.window if spec.chunk is None else spec.chunk,
+                      page_size=spec.page_size, v_head_dim=spec.v_head_dim)
 
     def cache_need(self):
         return self.need_of(self.spec)
@@ -169,12 +181,18 @@ class Attention:
         return decode_workspace(self.rt, batch, self.spec.num_heads, self.spec.head_dim)
 
     def _forward_prepared(self, x, batch, cache):
-        """The mixer without rotation and with any of: biases, a norm without weights, a factor on the queries that grows
-        with the position, values of their own width, keys and values of another run.  One kernel makes the heads ready
-        from the input product; the attention kernels are the same."""
+        """The mixer with any of: biases, a norm without weights, a factor on the queries that grows with the position,
+        values of their own width, keys and values of another run, chunks, the added one in the softmax's denominator,
+        values mixed with an earlier run's, a bias on the output.  One kernel makes the heads ready from the input product
+        (and turns them, where the mixer rotates); the attention kernels are the same."""
         s, rt = self.spec, self.rt
-        if self.position.rotary_table()[0] is not None:
-            raise NotImplementedError("an attention mixer with biases, a plain norm, a query factor or its own value width does not rotate")
+        from ..runtime import WeightedDelta
+        inv_freq, rotary_dim = self.position.rotary_table()
+        angles = None
+        if inv_freq is not None:
+            if getattr(self.position, "pairing", "half") != "half":
+                raise NotImplementedError("the kernel that makes these heads ready turns halves of a head, not neighbours")
+            angles = self.position.angles(batch)
         n = x.shape[0]
         table = batch.block_tables[cache.group]
         d, dv = s.head_dim, s.value_dim
@@ -184,29 +202,42 @@ class Attention:
         norm = "none" if s.qk_norm_eps is None else ("weighted" if s.qk_norm_weight else "plain")
         coef, every = s.q_temp if s.q_temp is not None else (0.0, 0)
         # (without projections of its own only q was projected: its columns stand at the row's start all the same)
-        fast = rt.dtype == "bfloat16" and d % 16 == 0 and d == dv \
+        fast = rt.dtype == "bfloat16" and d % 16 == 0 and d == dv and s.chunk is None and not s.sink \
             and rt.ops.attention_fast_ok(s.num_heads, s.num_kv_heads, cache.page_size, table.shape[1])
         capped = fast and s.softcap is not None
+        # mixed values: the source run leaves its values of this step's tokens for the runs that mix them in
+        v_in = v_out = None
+        if s.v_mix == "source":
+            v_out = batch.step_cache["attention_v_source"] = rt.empty((n, s.v_dim), torch.float32)
+        elif s.v_mix == "mix":
+            v_in = batch.step_cache.get("attention_v_source")
+            if v_in is None or tuple(v_in.shape) != (n, s.v_dim):
+                raise ValueError("an attention mixer that mixes values in runs behind the one whose values it reads, with values of the same sizes")
         q = rt.ops.head_prepare(proj, rt.empty((n, s.q_dim), rt.act_dtype), cache.k, cache.v, batch.positions,
                                 batch.seq_of_token, table, s.num_heads, s.num_kv_heads, d, dv, self.bias, norm,
                                 s.qk_norm_eps or 0.0, self.q_norm, self.k_norm, coef, every,
                                 write_kv=cache.writable and s.own_kv,
-                                q_head_scale=self.head_temp_capped if capped else self.head_temp, v_norm_eps=s.v_norm_eps)
+                                q_head_scale=self.head_temp_capped if capped else self.head_temp, v_norm_eps=s.v_norm_eps,
+                                angles=angles, rotary_dim=rotary_dim, v_first_in=v_in, v_first_out=v_out, v_lambda=self.v_lambda)
         if rt.dtype == "bfloat16" and not fast:
             rt.generic_attention_launches += 1
         out = rt.empty((n, s.out_dim), rt.act_dtype)
         paged_attention(rt, batch, q, out, cache.k, cache.v, cache.page_size, table, s.num_heads, s.num_kv_heads, d, dv,
-                        self.scale, s.window, fast, owner=self, softcap=s.softcap or 0.0)
-        return rt.linear(out, self.w_o, slabs=True, defer=True)
+                        self.scale, s.window, fast, owner=self, softcap=s.softcap or 0.0, chunk=s.chunk or 0, sink=s.sink)
+        delta = rt.linear(out, self.w_o, slabs=True, defer=True)
+        return delta if self.out_bias is None else WeightedDelta.of(rt, delta, 1.0, self.out_bias)
 
 
-def paged_attention(rt, batch, q, out, k_cache, v_cache, page_size, table, n_q, n_kv, d, dv, scale, window, fast, owner=None, softcap=0.0):
+def paged_attention(rt, batch, q, out, k_cache, v_cache, page_size, table, n_q, n_kv, d, dv, scale, window, fast, owner=None, softcap=0.0,
+                    chunk=0, sink=False):
     """The attention itself over a paged cache, for any mixer that has its queries ready: q [tokens, n_q d] -> out
     [tokens, n_q dv].  `fast`: the matrix-core kernels (prompt portions and single tokens each by their own; they
     need d == dv, or `v_cache` being `k_cache`, a value then being as wide as its key's row); else the generic kernel,
     which takes values of their own width (`v_cache` may be `k_cache` there too: a value is the first dv numbers
     of its key's row).  `softcap` c > 0: a scaled score s becomes c tanh(s / c) (with `fast`, q must come multiplied by scale / c).  `owner`: a mixer whose `_prefill_work(batch)` and `_workspace(batch)` make the work list and the
     decode workspace (else they are made here for these sizes)."""
+    if fast and (chunk or sink):
+        raise ValueError("the matrix-core attention kernels take a window, not chunks or an added one in the denominator")
     if fast:
         # capped scores: the builds that pass what they are given through tanh; q then comes times (scale / cap), and the cap is the scale
         capped = bool(softcap)
@@ -218,13 +249,13 @@ def paged_attention(rt, batch, q, out, k_cache, v_cache, page_size, table, n_q, 
             rt.ops.attention_decode(q, k_cache, v_cache, out, batch.decode_rows, batch.positions, batch.seq_of_token, table,
                                     n_q, n_kv, d, softcap if capped else scale, window or 0, batch.max_decode_ctx,
                                     owner._workspace(batch) if owner is not None else decode_workspace(rt, batch, n_q, d), capped=capped)
-    elif d == dv and v_cache is not k_cache and d <= 256 and not softcap:
+    elif d == dv and v_cache is not k_cache and d <= 256 and not softcap and not chunk and not sink:
         # the float32 path, and geometries the matrix-core kernels refuse (groups above 16, odd page sizes)
         rt.ops.paged_attention_generic(q, k_cache, v_cache, out, batch.positions, batch.seq_of_token, table, n_q, n_kv, d,
                                        scale, window or 0)
     else:
         rt.ops.paged_attention_wide(q, k_cache, v_cache, out, batch.positions, batch.seq_of_token, table, n_q, n_kv, d, dv,
-                                    scale, window or 0, softcap=softcap)
+                                    scale, window or 0, softcap=softcap, chunk=chunk, sink=sink)
     return out
 
 
@@ -289,3 +320,77 @@ def decode_workspace(rt, batch, num_heads, head_dim):
             ws = ws[:2]         # without the counts the splits are merged by a launch of its own
         batch.host[key] = ws
     return ws
+
+
+@register("mixer", "parallel_mixer")
+class ParallelMixer:
+    """Two mixers side by side on the same input (`ParallelMixerSpec`): delta = left_scale left(x) + right_scale right(x),
+    handed on as a weighted sum of the two results, which the block adds to the residual stream term by term.  One of them
+    may keep keys and values in pages and one a state of fixed size; each gets what it asked for."""
+
+    def __init__(self, spec, runtime):
+        from .base import part_class
+        self.spec = spec
+        self.rt = runtime
+        self.sides = [part_class("mixer", side.kind)(side, runtime) for side in (spec.left, spec.right)]
+        self.scales = (float(spec.left_scale), float(spec.right_scale))
+        self.graph_safe = all(getattr(side, "graph_safe", False) for side in self.sides)
+        if sum(side.cache_need() is not None for side in self.sides) > 1 or sum(side.state_need() is not None for side in self.sides) > 1:
+            raise ValueError("of two mixers side by side at most one keeps keys and values and at most one a state")
+
+    @staticmethod
+    def _side_classes(spec):
+        from .base import part_class
+        return [(side, part_class("mixer", side.kind)) for side in (spec.left, spec.right)]
+
+    @classmethod
+    def params(cls, spec):
+        out = {}
+        for side, side_cls in cls._side_classes(spec):
+            out.update({side.prefix + name: p for name, p in side_cls.params(side).items()})
+        return out
+
+    @classmethod
+    def placement(cls, spec):
+        out = {}
+        for side, side_cls in cls._side_classes(spec):
+            out.update({side.prefix + name: how for name, how in getattr(side_cls, "placement", lambda s: {})(side).items()})
+        return out
+
+    @classmethod
+    def variants(cls, spec, dtype):
+        out = []
+        for side, side_cls in cls._side_classes(spec):
+            for v in getattr(side_cls, "variants", lambda s, d: [])(side, dtype):
+                if v not in out:
+                    out.append(v)
+        return out
+
+    @classmethod
+    def need_of(cls, spec):
+        for side, side_cls in cls._side_classes(spec):
+            need = getattr(side_cls, "need_of", lambda s: None)(side)
+            if need is not None:
+                return need
+        return None
+
+    def load(self, tensors):
+        for side in self.sides:
+            prefix = side.spec.prefix
+            side.load({name[len(prefix):]: t for name, t in tensors.items() if name.startswith(prefix)})
+
+    def cache_need(self):
+        return next((need for need in (side.cache_need() for side in self.sides) if need is not None), None)
+
+    def state_need(self):
+        return next((need for need in (side.state_need() for side in self.sides) if need is not None), None)
+
+    def forward(self, x, batch, cache, state):
+        from ..runtime import WeightedDelta
+        total = None
+        for side, scale in zip(self.sides, self.scales):
+            delta = side.forward(x, batch, cache if side.cache_need() is not None else None, state if side.state_need() is not None else None)
+            term = WeightedDelta.of(self.rt, delta, scale)
+            total = term if total is None else total.plus(term)
+        return total
+

@@ -16,7 +16,7 @@ parts that do not say they take them.
 """
 from __future__ import annotations
 
-from ..runtime import Deferred, Pending
+from ..runtime import Deferred, Pending, WeightedDelta
 from .base import ParamSpec, register
 
 
@@ -53,6 +53,9 @@ class RMSNorm:
             if fused is not None:
                 return fused
             delta = delta.run()
+        elif isinstance(delta, WeightedDelta):
+            delta.add_to(x)         # every term where it lies, then the norm alone
+            return self.forward(x, out_dtype)
         elif isinstance(delta, Pending):
             delta = delta.run()
         return self.rt.ops.rmsnorm(x, self.weight, self.spec.eps, self.rt.empty(x.shape, out_dtype), delta=delta)

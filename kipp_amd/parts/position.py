@@ -92,6 +92,40 @@ class Rope:
         return table
 
 
+@register("position", "rope_band_scaled")
+class BandScaledRope(Rope):
+    """Rotary frequencies divided by `factor` where their wavelength is longer than original / low, kept where it is
+    shorter than original / high, and blended in between (`BandScaledRopeSpec` has the rule).  The table is computed
+    once in float64 and rounded to float32; the angle product is float32."""
+
+    def frequencies(self) -> torch.Tensor:
+        import math
+        s = self.spec
+        plain = super().frequencies()
+        out = plain.clone()
+        factor, low, high, original = float(s.factor), float(s.low), float(s.high), float(s.original)
+        for i, f in enumerate(plain.tolist()):
+            wavelength = 2.0 * math.pi / f
+            if wavelength < original / high:
+                continue
+            if wavelength > original / low:
+                out[i] = f / factor
+            else:
+                blend = (original / wavelength - low) / (high - low)
+                out[i] = (1.0 - blend) * f / factor + blend * f
+        return out
+
+    def angles(self, batch):
+        s = self.spec
+        key = ("rotary_angles_band", float(s.theta), self.rotary_dim, float(s.factor), float(s.low), float(s.high), float(s.original))
+        table = batch.step_cache.get(key)
+        if table is None:
+            table = self.rt.ops.rotary_angles(batch.positions, self.inv_freq,
+                                              self.rt.empty((batch.n_tokens, self.rotary_dim), torch.float32))
+            batch.step_cache[key] = table
+        return table
+
+
 @register("position", "rope_scaled")
 class ScaledRope(Rope):
     """Rotary frequencies stretched for contexts beyond the length a model was made for (`ScaledRopeSpec` has the

@@ -101,6 +101,39 @@ class Deferred(Pending):
         return self.rt.linear(self.x, self.w, slabs=self.slabs, x_steps_major=self.x_steps_major)
 
 
+class WeightedDelta(Pending):
+    """A weighted sum of deltas, each with the bias of the product that made it (or none): sum_i scale_i (delta_i + bias_i).
+    `terms`: (delta, scale, bias) with delta a tensor, slabs of one or another `Pending`.  `add_to(x)` adds every term to
+    the residual stream where it lies (one launch a term, nothing kept in between); `run()` gives the sum as a tensor."""
+    __slots__ = ("rt", "terms")
+
+    def __init__(self, rt, terms):
+        self.rt, self.terms = rt, [tuple(t) for t in terms]
+
+    @classmethod
+    def of(cls, rt, delta, scale=1.0, bias=None):
+        """`delta` times `scale` with `bias`; a weighted sum is taken apart rather than nested."""
+        if isinstance(delta, WeightedDelta) and bias is None:
+            return cls(rt, [(d, s * scale, b) for d, s, b in delta.terms])
+        return cls(rt, [(delta, float(scale), bias)])
+
+    def plus(self, other):
+        return WeightedDelta(self.rt, self.terms + WeightedDelta.of(self.rt, other).terms)
+
+    def add_to(self, x):
+        for delta, scale, bias in self.terms:
+            self.rt.ops.residual_add_scaled(x, self.rt.settle(delta), scale, bias)
+        return x
+
+    def run(self):
+        first = self.rt.settle(self.terms[0][0])
+        out = self.rt.ops.fill_zero(self.rt.empty(tuple(first.shape[-2:]), torch.float32))
+        self.rt.ops.residual_add_scaled(out, first, self.terms[0][1], self.terms[0][2])
+        for delta, scale, bias in self.terms[1:]:
+            self.rt.ops.residual_add_scaled(out, self.rt.settle(delta), scale, bias)
+        return out
+
+
 class Runtime:
     FUSE_NORM_X_BYTES = 40e6    # most bytes of X the workgroups of an unsplit product may read together for the fused norm to pay
 
