@@ -1,0 +1,526 @@
+"""The Zivazen design on the GPU against its plain implementation: every new kernel alone (crafted inputs at the edges),
+then the engine under every cutting in both precisions, tight pools, slots used again, long decoding, recorded steps,
+other sizes, generation through the scheduler, the trace replay and the command line."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from tests import helpers as H
+from tests.plain import zivazen_plain as P
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SHAPES = ("zivazen-tiny-a", "zivazen-tiny-b")
+LENGTHS = [1, 19, 45, 80, 131]
+TOL = {"float32": 1e-9, "bfloat16": 3e-2}     # float32 is the sharp test; at these narrow widths bfloat16 rows are noisy and a close call of a router may fall the other way
+
+
+def sharpen(folder, factor=6.0):
+    """Larger query and key matrices in the attention layers, so that few keys carry a row's softmax and a key that is
+    wrongly seen or missed shows in the logits."""
+    from safetensors import safe_open
+    from safetensors.torch import save_file
+    path = os.path.join(folder, "model.safetensors")
+    tensors = {}
+    with safe_open(path, framework="pt") as f:
+        for name in f.keys():
+            tensors[name] = f.get_tensor(name)
+    for name in list(tensors):
+        if name.endswith((".mix.q", ".mix.k", ".mix.left.q", ".mix.left.k", ".mix.q.norm")):
+            tensors[name] = (tensors[name].float() * (factor if "left" in name or name.endswith("norm") else 1.0)).to(tensors[name].dtype)
+    save_file(tensors, path)
+    return folder
+
+
+def write_model(path, cfg, seed, dtype):
+    from kipp_amd.weights import write_random_model
+    return sharpen(write_random_model(str(path), cfg, seed=seed, dtype=dtype))
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    from kipp_amd.config import shape_config
+    root = tmp_path_factory.mktemp("zivazen")
+    return {(shape, dtype): write_model(root / f"{shape}-{dtype}", shape_config(shape), 50 + i, dtype)
+            for i, shape in enumerate(SHAPES) for dtype in ("float32", "bfloat16")}
+
+
+_plain_cache = {}
+_margin_cache = {}
+
+
+def plain_logits(folder, tokens):
+    key = (folder, tuple(tokens))
+    if key not in _plain_cache:
+        cfg, w = P.load_folder(folder)
+        margins = []
+        _plain_cache[key] = P.forward_whole(cfg, w, list(tokens), margins=margins)
+        routed = sum(1 for layer in cfg["layers"] if (layer.get("mlp") or {}).get("kind") == "moe")
+        _margin_cache[id(_plain_cache[key])] = np.min(np.array(margins).reshape(routed, len(tokens)), axis=0) if routed else None
+    return _plain_cache[key]
+
+
+FLIPS = 0.5         # share of a request's positions that may lie beyond the bfloat16 bound (see `close`)
+CLOSE_CALL = 0.02   # a router's margin (in choice scores) below which bfloat16 rows may choose another expert
+
+
+def close(got, ref, tol, what):
+    """Every position's normalised squared error within `tol`.  Under the bfloat16 bound a router's choice between two
+    experts whose scores differ by less than the rounding of the rows it reads falls either way, and the position (and,
+    through the state space layers, every one after it) then differs by much more than rounding: a request passes if every
+    position beyond the bound stands at or behind a close call of the plain implementation's routers, or if no more than a
+    share of its positions lie beyond it.  The float32 runs of the same cases allow no such position."""
+    assert got.shape == ref.shape and np.isfinite(got).all(), what
+    each = [float(np.sum((g - r) ** 2) / np.sum(r ** 2)) for g, r in zip(got.astype(np.float64), ref)]
+    errs = sorted(each)
+    spared = int(FLIPS * len(errs)) if tol >= TOL["bfloat16"] else 0
+    margins = _margin_cache.get(id(ref)) if spared else None
+    if margins is not None and len(margins) == len(each):
+        called = np.minimum.accumulate(margins) < CLOSE_CALL
+        if all(e <= tol or c for e, c in zip(each, called)):
+            return
+    worst = errs[len(errs) - 1 - spared]
+    over = sum(e > tol for e in errs)
+    assert worst <= tol, f"{what}: NMSE {worst:.3e} exceeds {tol:.1e} ({over} of {len(errs)} positions beyond it, {spared} spared)"
+
+
+def engine_of(folder, dtype, page=16, **kw):
+    from kipp_amd.engine import Engine
+    kw.setdefault("max_tokens", 1024)
+    return Engine.from_folder(folder, dtype=dtype, page_size=page, share_prefixes=False, **kw)
+
+
+def dev(a, ty=None):
+    import torch
+    return None if a is None else torch.tensor(np.asarray(a), device="cuda:0", dtype=ty)
+
+
+def f32(a):
+    import torch
+    return dev(np.asarray(a, dtype=np.float32), torch.float32)
+
+
+def i32(a):
+    import torch
+    return dev(np.asarray(a, dtype=np.int32), torch.int32)
+
+
+def requests_of(vocab, seed=0, lengths=LENGTHS):
+    return {f"r{i}": H.random_tokens(seed * 100 + i, n, vocab) for i, n in enumerate(lengths)}
+
+
+def _entries(lengths, slots):
+    starts = np.concatenate([[0], np.cumsum(lengths)[:-1]])
+    seq_of = np.concatenate([np.full(n, i) for i, n in enumerate(lengths)])
+    return i32(starts), i32(lengths), i32(slots), i32(seq_of), starts
+
+
+# =============================================================================== the kernels alone
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H_, G, d, dv, rot, chunk, page", [(4, 2, 32, 16, 16, 40, 16), (6, 2, 24, 24, 24, 11, 8), (3, 3, 96, 48, 2, 17, 16),
+                                                           (2, 1, 200, 80, 64, 64, 32), (2, 2, 16, 16, 8, 1, 16), (8, 2, 64, 32, 64, 150, 16)])
+def test_prepared_heads_and_chunked_attention_with_a_key_that_stands_out(dtype, H_, G, d, dv, rot, chunk, page):
+    """Biases, weighted head norms, the rotation over part of the head, mixed values, chunks and the added one against the
+    plain functions on random inputs; then one key whose score stands out: first of the last row's chunk, last of the chunk
+    before, at a page border inside the chunk, far back, the row itself: seen by the last row of a prompt portion and by a
+    single token exactly when the design says so."""
+    import torch
+    from kipp_amd.csrc import ops
+    ty = torch.float32 if dtype == "float32" else torch.bfloat16
+    rng = np.random.default_rng(d + chunk)
+    T, scale, eps, lam = 150, 0.3, 1e-5, 0.35
+    freq = P.rotary_frequencies(rot, 5000.0, {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 64})
+    pages = -(-T // page)
+    order = rng.permutation(pages + 3)[:pages]
+    table = i32(order.reshape(1, pages))
+    positions, seq_of = i32(np.arange(T)), i32(np.zeros(T))
+    angles = ops.rotary_angles(positions, f32(freq), torch.empty((T, rot), device="cuda:0"))
+    bias = rng.normal(size=H_ * d + G * d + G * dv).astype(np.float32) * 0.3
+    qw, kw = rng.uniform(0.5, 1.5, size=d).astype(np.float32), rng.uniform(0.5, 1.5, size=d).astype(np.float32)
+    v_first = rng.normal(size=(T, G * dv)).astype(np.float32)
+
+    def run(proj, rows, use_bias=True, norm="weighted"):
+        kc = torch.zeros((pages + 3, G, page, d), dtype=ty, device="cuda:0")
+        vc = torch.zeros((pages + 3, G, page, dv), dtype=ty, device="cuda:0")
+        kept = torch.empty((T, G * dv), device="cuda:0")
+        q = ops.head_prepare(f32(proj), torch.empty((T, H_ * d), dtype=ty, device="cuda:0"), kc, vc, positions, seq_of, table, H_, G, d, dv,
+                             f32(bias) if use_bias else None, norm, eps, f32(qw), f32(kw), angles=angles, rotary_dim=rot,
+                             v_first_in=f32(v_first), v_first_out=kept, v_lambda=f32([lam]))
+        idx = np.asarray(rows)
+        out = torch.empty((len(idx), H_ * dv), dtype=ty, device="cuda:0")
+        ops.paged_attention_wide(q[dev(idx, torch.int64)].contiguous(), kc, vc, out, i32(idx), i32(np.zeros(len(idx))), table, H_, G, d, dv, scale,
+                                 chunk=chunk, sink=True)
+        return out.float().cpu().numpy().reshape(len(idx), H_, dv), kept.cpu().numpy()
+
+    proj = rng.normal(size=(T, H_ * d + G * d + G * dv)).astype(np.float32)
+    p64 = proj.astype(np.float64) + bias.astype(np.float64)
+    pos = list(range(T))
+    q = P.rotate(P.rms_norm(p64[:, :H_ * d].reshape(T, H_, d), qw, eps), pos, rot, freq)
+    k = P.rotate(P.rms_norm(p64[:, H_ * d:H_ * d + G * d].reshape(T, G, d), kw, eps), pos, rot, freq)
+    v_own = p64[:, H_ * d + G * d:]
+    v = ((1 - lam) * v_own + lam * v_first).reshape(T, G, dv)
+    ref = P.attention_core(q, k, v, scale, lambda i, j: i // chunk == j // chunk, sink=True)
+    tol = 2e-4 if dtype == "float32" else 6e-2
+    got, kept = run(proj, range(T))
+    assert np.allclose(kept, v_own, rtol=1e-5, atol=1e-5)
+    assert np.allclose(got, ref, rtol=tol, atol=tol)
+    # one key stands out (no bias, no norm weight games: unit directions; the rotation turns query and key alike only at
+    # equal positions, so the standing-out pair is built from the numbers the rotation leaves alone where there are any)
+    if rot == d:
+        return
+    u = np.zeros(d, dtype=np.float32)
+    u[rot:] = rng.normal(size=d - rot)
+    u /= np.linalg.norm(u)
+    last = T - 1
+    start = last - last % chunk
+    for key, seen in ((start, True), (start - 1, False), (0, start == 0), (-(-start // page) * page, True), (last, True)):
+        if key < 0 or key > last:
+            continue
+        seen = seen and key >= start
+        crafted = proj.copy()
+        crafted[:, H_ * d:H_ * d + G * d] = np.tile(-60.0 * u, G)
+        crafted[last, :H_ * d] = np.tile(60.0 * u, H_)
+        crafted[key, H_ * d:H_ * d + G * d] = np.tile(60.0 * u, G)
+        crafted[:, H_ * d + G * d:] = 0.0
+        crafted[key, H_ * d + G * d::dv] = 50.0
+        for rows in (range(T), [last]):
+            out = run(crafted, rows, use_bias=False, norm="plain")[0][-1]
+            mixed = (1 - lam) * 50.0 + lam * v_first[key].reshape(G, dv)[:, 0]        # the value that was cached for the key
+            want = np.repeat(mixed, H_ // G)
+            if seen:
+                assert np.allclose(out[:, 0], want, rtol=3e-2, atol=0.3), (key, list(rows)[:2], out[:, 0], want)
+            else:
+                assert np.all(np.abs(out[:, 0]) < 0.5 * np.abs(want)), (key, list(rows)[:2], out[:, 0])
+
+
+@pytest.mark.parametrize("heads, groups, n, p, taps, parts", [(4, 2, 16, 24, 3, 2), (6, 3, 64, 32, 4, 1), (2, 2, 36, 20, 2, 4), (3, 1, 130, 8, 1, 3),
+                                                             (2, 1, 600, 16, 5, 1), (1, 1, 8, 260, 16, 1), (8, 1, 128, 64, 4, 8)])
+def test_state_space_kernels_across_cuts(heads, groups, n, p, taps, parts):
+    """Three entries of unequal length in slots of any order, then their next tokens (single tokens, then the rest as
+    portions) from the kept states and the filters' kept inputs: prepare, walk and finish against the plain walk over the
+    whole sequences."""
+    import torch
+    from kipp_amd.csrc import ops
+    rng = np.random.default_rng(heads * 1000 + n)
+    inner, gn = heads * p, groups * n
+    channels = inner + 2 * gn
+    width = inner + channels + heads + 3
+    conv_w, conv_b = rng.normal(size=(channels, taps)).astype(np.float32) * 0.5, rng.normal(size=channels).astype(np.float32) * 0.1
+    a_log, dt_bias, skip = (rng.normal(size=heads).astype(np.float32) * 0.5 for _ in range(3))
+    norm_w = rng.uniform(0.5, 1.5, size=inner).astype(np.float32)
+    totals, first = [23, 7, 40], [17, 6, 1]
+    seqs = [rng.normal(size=(t, width)).astype(np.float32) for t in totals]
+    size = ops.ssd_state_size(heads, groups, n, p, taps)
+    state = torch.zeros((6, size), device="cuda:0")
+    slots = [4, 0, 2]
+    got = [[] for _ in totals]
+    eps = 1e-5
+    for part in (0, 1, 2):
+        lengths = [first[i] if part == 0 else (1 if part == 1 else totals[i] - first[i] - 1) for i in range(3)]
+        at = [0 if part == 0 else (first[i] if part == 1 else first[i] + 1) for i in range(3)]
+        live = [i for i in range(3) if lengths[i] > 0]
+        proj = f32(np.concatenate([seqs[i][at[i]:at[i] + lengths[i]] for i in live]))
+        qs, ql, sl, seq_of, starts = _entries([lengths[i] for i in live], [slots[i] for i in live])
+        rows = proj.shape[0]
+        prep = torch.empty((rows, ops.ssd_prep_width(heads, groups, n, p)), device="cuda:0")
+        ops.ssd_prepare(proj, f32(conv_w), f32(conv_b), f32(a_log), f32(dt_bias), state, seq_of, qs, ql, sl, prep, heads, groups, n, p)
+        o = ops.gated_scan(prep, state, qs, ql, sl, torch.empty((rows, inner), device="cuda:0"), heads, groups, n, p, longest=max(lengths))
+        out = ops.ssd_finish(o, prep, 2 * gn + inner, proj, 0, f32(skip), p, f32(norm_w), eps, inner // parts, torch.empty((rows, inner), device="cuda:0"))
+        out = out.cpu().numpy()
+        for j, i in enumerate(live):
+            got[i].append(out[starts[j]:starts[j] + lengths[i]])
+    for i, t in enumerate(totals):
+        s = seqs[i].astype(np.float64)
+        z = s[:, :inner]
+        xbc = P.silu(P.causal_filter(s[:, inner:inner + channels], conv_w, conv_b))
+        dt = P.softplus(s[:, inner + channels:inner + channels + heads] + dt_bias.astype(np.float64))
+        y, S = P.ssd_scan(xbc[:, :inner].reshape(t, heads, p), xbc[:, inner:inner + gn].reshape(t, groups, n),
+                          xbc[:, inner + gn:].reshape(t, groups, n), dt, a_log.astype(np.float64), skip.astype(np.float64))
+        gated = y.reshape(t, inner) * P.silu(z)
+        ref = P.rms_norm(gated.reshape(t, parts, inner // parts), None, eps).reshape(t, inner) * norm_w
+        out = np.concatenate(got[i])
+        assert np.allclose(out, ref, rtol=5e-4, atol=5e-4 * np.abs(ref).max()), (i, np.abs(out - ref).max())
+        kept = state[slots[i], :heads * n * p].cpu().numpy().reshape(heads, p, n)
+        assert np.allclose(kept, S.transpose(0, 2, 1), rtol=5e-4, atol=5e-4 * np.abs(S).max())
+        if taps > 1:
+            tail = state[slots[i], heads * n * p:heads * n * p + (taps - 1) * channels].cpu().numpy().reshape(taps - 1, channels)
+            want = np.concatenate([np.zeros((taps - 1, channels)), s[:, inner:inner + channels]])[-(taps - 1):]
+            assert np.allclose(tail, want, atol=1e-6)
+    assert float(state[[1, 3, 5]].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("experts, top, count, keep, tokens", [(16, 2, 4, 2, 37), (12, 2, 4, 3, 300), (6, 3, 3, 2, 1), (8, 1, 1, 1, 20), (64, 8, 8, 4, 129),
+                                                               (9, 9, 1, 1, 5), (130, 4, 65, 3, 40), (10, 2, 10, 2, 33)])
+def test_grouped_router(experts, top, count, keep, tokens):
+    """Sigmoid scores, the correction in the choice but not in the weights, groups of which the best stay (a group of one
+    counts its one score), the scale; exact ties and an expert whose correction alone lifts it."""
+    import torch
+    from kipp_amd.csrc import ops
+    rng = np.random.default_rng(experts * 7 + top)
+    z = rng.normal(size=(tokens, experts + 3)).astype(np.float32) * 2
+    corr = rng.normal(size=experts).astype(np.float32) * 0.3
+    corr[experts // 2] = 2.0
+    if tokens > 3:
+        z[3, :experts] = 0.25           # every score equal: the correction and then the index decide
+    chosen = torch.empty((tokens, top), dtype=torch.int32, device="cuda:0")
+    weight = torch.empty((tokens, top), device="cuda:0")
+    pair_token = torch.empty((tokens * top,), dtype=torch.int32, device="cuda:0")
+    place = torch.empty((tokens * top,), dtype=torch.int32, device="cuda:0")
+    tiles = torch.empty((ops.moe_max_tiles(tokens, experts, top), 3), dtype=torch.int32, device="cuda:0")
+    ops.moe_route(f32(z), experts, top, 1e-20, chosen, weight, pair_token, place, tiles, router="sigmoid", correction=f32(corr), groups=(count, keep), scale=2.5)
+    chosen, weight = chosen.cpu().numpy(), weight.cpu().numpy()
+    for t in range(tokens):
+        ref_e, ref_w, margin = P.route(z[t, :experts].astype(np.float64), corr.astype(np.float64), top, count, keep, 2.5)
+        if margin < 1e-5:
+            assert sorted(chosen[t]) == sorted(set(chosen[t])) and np.isclose(weight[t].sum(), 2.5, rtol=1e-4)
+            if t != 3:
+                continue
+        assert list(chosen[t]) == ref_e, (t, chosen[t], ref_e)
+        assert np.allclose(weight[t], ref_w, rtol=1e-5)
+    # the sorted pairs cover every (token, choice) once
+    assert sorted(place.cpu().numpy().tolist()) == list(range(tokens * top))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_squared_relu_experts_biased_activation_and_the_weighted_sum(dtype):
+    import torch
+    from kipp_amd.csrc import ops
+    ty = torch.float32 if dtype == "float32" else torch.bfloat16
+    rng = np.random.default_rng(5)
+    u = rng.normal(size=(3, 21, 2 * 40)).astype(np.float32)
+    bias = rng.normal(size=80).astype(np.float32)
+    out = ops.activate(f32(u), torch.empty((21, 40), dtype=ty, device="cuda:0"), "silu", glu=True, bias=f32(bias)).float().cpu().numpy()
+    total = u.astype(np.float64).sum(0) + bias
+    ref = P.silu(total[:, :40]) * total[:, 40:]
+    assert np.allclose(out, ref, rtol=1e-5 if dtype == "float32" else 1e-2, atol=1e-5 if dtype == "float32" else 2e-2)
+    out = ops.activate(f32(u[:1, :, :40].copy()), torch.empty((21, 40), dtype=ty, device="cuda:0"), "relu2").float().cpu().numpy()
+    assert np.allclose(out, np.maximum(u[0, :, :40], 0) ** 2, rtol=1e-2, atol=1e-6)
+    x = rng.normal(size=(21, 40)).astype(np.float32)
+    delta = rng.normal(size=(2, 21, 40)).astype(np.float32)
+    b = rng.normal(size=40).astype(np.float32)
+    got = ops.residual_add_scaled(f32(x), f32(delta), 1.3, f32(b)).cpu().numpy()
+    assert np.allclose(got, x + 1.3 * (delta.sum(0) + b), rtol=1e-6, atol=1e-6)
+    got = ops.residual_add_scaled(f32(x), f32(delta[0]), -0.5).cpu().numpy()
+    assert np.allclose(got, x - 0.5 * delta[0], rtol=1e-6, atol=1e-6)
+
+
+# =============================================================================== the engine
+
+@pytest.mark.parametrize("dtype, page", [("float32", 16), ("bfloat16", 16), ("bfloat16", 32), ("float32", 8)])
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("cut", ["whole", "tail", "portions", "mixed"])
+def test_cuttings_match_plain(folders, shape, dtype, page, cut):
+    """Whole prompts, the last tokens one by one, portions of changing size down to two tokens, and mixed batches in a
+    pool that only holds the live requests and has four state slots (pages and slots are used again)."""
+    folder = folders[(shape, dtype)]
+    vocab = P.load_folder(folder)[0]["vocab"]
+    requests = requests_of(vocab)
+    if cut == "mixed":
+        requests.update({f"s{i}": H.random_tokens(900 + i, n, vocab) for i, n in enumerate(LENGTHS)})
+        steps = H.mixed(requests, seed=5)
+        engine = engine_of(folder, dtype, page, max_tokens=None, num_pages=H.peak_pages(requests, steps, page), max_requests=4)
+    else:
+        engine = engine_of(folder, dtype, page)
+        steps = {"whole": H.whole, "tail": H.tail_one_by_one, "portions": H.changing_portions}[cut](requests)
+    got = H.replay(engine, requests, steps)
+    for rid, toks in requests.items():
+        close(got[rid], plain_logits(folder, toks), TOL[dtype], f"{shape}/{dtype}/{page}/{cut}/{rid}")
+    assert engine.cache.free_pages() == [g.pool.num_pages for g in engine.cache.groups]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_float32_cuttings_are_bitwise_equal(folders, shape):
+    """In float32 every sum runs in an order that the token's own position fixes: how the prompt was cut, what else was
+    in the batch and which pages and slots were used change no bit."""
+    folder = folders[(shape, "float32")]
+    requests = requests_of(P.load_folder(folder)[0]["vocab"], seed=3)
+    base = H.replay(engine_of(folder, "float32"), requests, H.whole(requests))
+    for maker in (H.tail_one_by_one, H.changing_portions, lambda r: H.mixed(r, seed=11)):
+        steps = maker(requests)
+        order = list(np.random.default_rng(1).permutation(64))
+        got = H.replay(engine_of(folder, "float32", page_order=order, max_requests=5), requests, steps)
+        for rid in requests:
+            assert np.array_equal(got[rid], base[rid]), f"{shape}/{rid}: bits differ between cuttings"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_through_a_small_pool_and_one_slot(tmp_path, dtype):
+    """A window of 20 and chunks of 24 in pages of 16 beside the state space layer: 200 tokens pass through the few pages
+    that the window and the chunk need and the one state slot, which a second request then takes over (its state and its
+    filter's last inputs must start at zero, not where the first left them)."""
+    cfg = {"architecture": "Zivazen", "vocab": 90, "width": 64, "norm": {"eps": 1e-5},
+           "layers": [{"type": "parallel", "mixer": {"left": {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 16, "scale": 0.25, "mask": {"size": 20},
+                                                              "rot": {"base": 100.0, "dims": 8}},
+                                                     "right": {"heads": 2, "vdim": 16, "state": 24, "groups": 1, "conv": 4, "norm_groups": 1},
+                                                     "left_scale": 1.0, "right_scale": 0.5}, "mlp": {"kind": "dense", "ff": 48}},
+                      {"type": "attention", "mixer": {"heads": 4, "kv_heads": 1, "dim": 16, "vdim": 8, "scale": 0.25, "mask": {"size": 24},
+                                                      "rot": {"base": 50.0, "dims": 16, "scaling": {"factor": 2.0, "low": 1.0, "high": 2.0, "original": 32}}, "v_mix": True},
+                       "mlp": {"kind": "moe", "router": {"experts": 4, "top": 2, "groups": {"count": 2, "keep": 1}, "scale": 1.0}, "expert": {"ff": 32}, "shared": {"ff": 32}}},
+                      {"type": "attention", "mixer": {"heads": 4, "kv_heads": 1, "dim": 32, "vdim": 8, "scale": 0.2, "mask": {"size": 7},
+                                                      "rot": {"base": 50.0, "dims": 4}, "v_mix": True}, "mlp": None}]}
+    folder = write_model(tmp_path / "three", cfg, 8, dtype)
+    tokens = {"r": H.random_tokens(77, 200, 90), "next": H.random_tokens(78, 40, 90)}
+    engine = engine_of(folder, dtype, 16, max_tokens=None, num_pages=4, max_requests=1)
+    steps = [([("r", 10)], [])] + [([("r", 1)], []) for _ in range(60)] + [([("r", 7)], []), ([("r", 2)], [])] \
+        + [([("r", 1)], []) for _ in range(121)]
+    steps[-1] = (steps[-1][0], ["r"])
+    steps += [([("next", 33)], [])] + [([("next", 1)], []) for _ in range(7)]
+    steps[-1] = (steps[-1][0], ["next"])
+    got = H.replay(engine, tokens, steps)
+    for rid in tokens:
+        close(got[rid], plain_logits(folder, tokens[rid]), TOL[dtype], f"four pages/{dtype}/{rid}")
+    if dtype == "bfloat16":
+        assert engine.graphs.replays > 100          # the single tokens ran as recorded steps
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_other_sizes_and_branches(tmp_path, dtype):
+    """Widths that are no multiple of 8 or of 32, a window and a chunk of one, a window and a chunk longer than the prompt,
+    eighteen heads on one key/value head, a head that turns whole, a state of 260 numbers, one tap, one group of one expert,
+    every expert chosen, layers of one kind only, scales of one; prompts of more rows than the few-rows products take."""
+    att = lambda heads, kv, dim, vdim, size, dims, **more: dict({"heads": heads, "kv_heads": kv, "dim": dim, "vdim": vdim, "scale": 0.2, "mask": {"size": size},
+                                                                 "rot": {"base": 300.0, "dims": dims}}, **more)
+    ssd = lambda heads, vdim, state, groups, conv, parts: {"heads": heads, "vdim": vdim, "state": state, "groups": groups, "conv": conv, "norm_groups": parts}
+    layers = [
+        {"type": "attention", "mixer": att(18, 1, 16, 16, 1, 16), "mlp": None},
+        {"type": "parallel", "mixer": {"left": att(2, 2, 40, 24, 1, 2), "right": ssd(1, 20, 260, 1, 1, 1), "left_scale": 1.0, "right_scale": 1.0},
+         "mlp": {"kind": "dense", "ff": 30}},
+        {"type": "attention", "mixer": att(4, 2, 32, 32, 1000, 8, v_mix=True),
+         "mlp": {"kind": "moe", "router": {"experts": 1, "top": 1, "groups": {"count": 1, "keep": 1}, "scale": 1.0}, "expert": {"ff": 20}}},
+        {"type": "parallel", "mixer": {"left": att(3, 3, 32, 32, 1000, 32), "right": ssd(12, 4, 8, 4, 7, 6), "left_scale": 0.25, "right_scale": 2.0}, "mlp": None},
+        {"type": "attention", "mixer": att(2, 2, 32, 32, 300, 32, v_mix=True),
+         "mlp": {"kind": "moe", "router": {"experts": 9, "top": 9, "groups": {"count": 3, "keep": 3}, "scale": 0.5}, "expert": {"ff": 8}, "shared": {"ff": 100}}}]
+    for width, chosen in ((100, layers), (72, [layers[0], layers[2], layers[4]]), (64, [layers[1], layers[3]])):
+        cfg = {"architecture": "Zivazen", "vocab": 77, "width": width, "norm": {"eps": 1e-6}, "layers": chosen}
+        folder = write_model(tmp_path / f"odd{width}", cfg, width, dtype)
+        requests = {"long": H.random_tokens(1, 330, 77), "short": H.random_tokens(2, 9, 77)}
+        for steps in (H.whole(requests), [([("long", 270)], []), ([("long", 59), ("short", 8)], []), ([("long", 1), ("short", 1)], ["long", "short"])]):
+            got = H.replay(engine_of(folder, dtype), requests, steps)
+            for rid, toks in requests.items():
+                close(got[rid], plain_logits(folder, toks), TOL[dtype] * (4 if dtype == "bfloat16" else 1), f"{width}/{dtype}/{rid}")
+
+
+def random_configuration(rng):
+    """A model of the design with every size, the order of its layers and every constant drawn at random."""
+    def rotation(d):
+        rot = {"base": rng.choice([100.0, 10000.0, 500000.0]), "dims": rng.choice([n for n in (2, 8, 16, 32, 64, 96) if n <= d])}
+        if rng.random() < 0.5:
+            rot["scaling"] = {"factor": rng.choice([2.0, 8.0]), "low": 1.0, "high": rng.choice([2.0, 4.0]), "original": rng.choice([16, 64, 256])}
+        return rot
+    layers = []
+    mix_sizes = (rng.choice([1, 2]), rng.choice([16, 24, 64]))
+    for i in range(rng.randint(3, 6)):
+        kind = rng.choice(["attention", "parallel"])
+        r = rng.random()
+        if r < 0.15:
+            mlp = None
+        elif r < 0.55:
+            mlp = {"kind": "dense", "ff": rng.choice([128, 200, 384])}
+        else:
+            count = rng.choice([1, 2, 4])
+            size = rng.choice([1, 2, 3])
+            keep = rng.randint(1, count)
+            mlp = {"kind": "moe", "router": {"experts": count * size, "top": rng.randint(1, min(4, keep * size)), "groups": {"count": count, "keep": keep},
+                                             "scale": rng.choice([1.0, 2.5])}, "expert": {"ff": rng.choice([24, 64, 100])}}
+            if rng.random() < 0.6:
+                mlp["shared"] = {"ff": rng.choice([32, 72])}
+        if kind == "attention":
+            mixes = rng.random() < 0.7
+            groups = mix_sizes[0] if mixes else rng.choice([1, 2, 3])
+            d = rng.choice([16, 32, 40, 64, 96])
+            mixer = {"heads": groups * rng.choice([1, 2, 3]), "kv_heads": groups, "dim": d, "vdim": mix_sizes[1] if mixes else rng.choice([16, d]),
+                     "scale": rng.uniform(0.05, 0.3), "mask": {"size": rng.choice([1, 5, 16, 17, 64, 100, 300])}, "rot": rotation(d)}
+            if mixes:
+                mixer["v_mix"] = True
+        else:
+            groups = rng.choice([1, 2, 4])
+            d = rng.choice([16, 32, 48, 64])
+            left = {"heads": groups * rng.choice([1, 2, 3]), "kv_heads": groups, "dim": d, "vdim": d if rng.random() < 0.6 else rng.choice([16, 24, 64]),
+                    "scale": rng.uniform(0.05, 0.3), "mask": {"size": rng.choice([1, 5, 16, 17, 64, 100, 300])}, "rot": rotation(d)}
+            sg = rng.choice([1, 2])
+            heads = sg * rng.choice([1, 2, 3])
+            p = rng.choice([8, 16, 40])
+            right = {"heads": heads, "vdim": p, "state": rng.choice([8, 16, 48, 130]), "groups": sg, "conv": rng.choice([1, 2, 4, 7]),
+                     "norm_groups": rng.choice([1, heads])}
+            mixer = {"left": left, "right": right, "left_scale": rng.choice([1.0, 0.6, 1.2]), "right_scale": rng.choice([1.0, 1.1, 0.3])}
+        layers.append({"type": kind, "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Zivazen", "vocab": rng.choice([300, 512]), "width": rng.choice([96, 128, 192]),
+            "norm": {"eps": rng.choice([1e-5, 1e-6])}, "layers": layers}
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_models_drawn_at_random(tmp_path, seed):
+    """Sizes, order of layers and constants drawn at random; whole prompts, portions and mixed batches in float32."""
+    import random
+    cfg = random_configuration(random.Random(seed))
+    folder = write_model(tmp_path / "drawn", cfg, seed, "float32")
+    requests = {f"r{i}": H.random_tokens(seed * 10 + i, n, cfg["vocab"]) for i, n in enumerate([1, 23, 97, 180])}
+    for maker in (H.whole, H.changing_portions, lambda r: H.mixed(r, seed=seed)):
+        got = H.replay(engine_of(folder, "float32", max_requests=4), requests, maker(requests))
+        for rid, toks in requests.items():
+            close(got[rid], plain_logits(folder, toks), 2e-8, f"drawn {seed}/{rid}: {json.dumps(cfg)}")
+
+
+def test_recorded_steps_of_a_changing_batch(folders):
+    """Three requests decode together from recorded steps while window and chunk pass page borders and the state goes on
+    in its slot; one ends early and the batch goes on at another size."""
+    folder = folders[("zivazen-tiny-a", "bfloat16")]
+    vocab = P.load_folder(folder)[0]["vocab"]
+    requests = {"a": H.random_tokens(1, 90, vocab), "b": H.random_tokens(2, 120, vocab), "c": H.random_tokens(3, 75, vocab)}
+    engine = engine_of(folder, "bfloat16")
+    steps = [([("a", 30), ("b", 51), ("c", 2)], [])]
+    fed = {"a": 30, "b": 51, "c": 2}
+    while any(fed[r] < len(requests[r]) for r in fed):
+        live = [r for r in fed if fed[r] < len(requests[r])]
+        for r in live:
+            fed[r] += 1
+        steps.append(([(r, 1) for r in live], [r for r in live if fed[r] == len(requests[r])]))
+    got = H.replay(engine, requests, steps)
+    for rid, toks in requests.items():
+        close(got[rid], plain_logits(folder, toks), TOL["bfloat16"], f"recorded/{rid}")
+    assert engine.graphs.replays > 50
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_scheduler(folders, dtype):
+    """`generate` (scheduler, continuous batching, tokens chosen on the device) against the plain implementation:
+    every generated token is the plain argmax of its position, or within rounding of it."""
+    from kipp_amd import generate
+    folder = folders[("zivazen-tiny-b", dtype)]
+    cfg, w = P.load_folder(folder)
+    prompts = [H.random_tokens(5, 3, cfg["vocab"]), H.random_tokens(6, 40, cfg["vocab"]), H.random_tokens(7, 21, cfg["vocab"])]
+    outputs = generate(folder, prompts, max_new_tokens=30, dtype=dtype, page_size=16, prefill_chunk=16, max_step_tokens=24)
+    margin = 1e-4 if dtype == "float32" else 0.05
+    for prompt, out in zip(prompts, outputs):
+        assert len(out) == 30
+        logits = P.forward_whole(cfg, w, prompt + out)
+        for i, tok in enumerate(out):
+            row = logits[len(prompt) - 1 + i]
+            assert row[tok] >= row.max() - margin * (row.max() - row.min()), (dtype, i)
+
+
+def test_trace_replay_and_command_line(folders, tmp_path):
+    folder = folders[("zivazen-tiny-a", "bfloat16")]
+    vocab = P.load_folder(folder)[0]["vocab"]
+    toks = H.random_tokens(4, 60, vocab)
+    lines = [{"step": 0, "entries": [{"id": "x", "tokens": toks[:33], "want": [0, 32]}], "end": []},
+             {"step": 1, "entries": [{"id": "x", "tokens": toks[33:35], "want": []}, {"id": "y", "tokens": toks[:7], "want": [6]}], "end": ["y"]},
+             {"step": 2, "entries": [{"id": "x", "tokens": toks[35:36], "want": [0]}], "end": ["x"]}]
+    out = tmp_path / "out"
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", "bfloat16", "--out", str(out),
+                          "--max-tokens", "128"], input="\n".join(json.dumps(l) for l in lines) + "\n", capture_output=True, text=True, timeout=600)
+    assert run.returncode == 0, run.stderr[-2000:]
+    assert [l for l in run.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    ref = plain_logits(folder, toks)
+    close(np.fromfile(out / "0.f32", dtype="<f4").reshape(2, vocab), ref[[0, 32]], TOL["bfloat16"], "trace step 0")
+    close(np.fromfile(out / "1.f32", dtype="<f4").reshape(1, vocab), ref[[6]], TOL["bfloat16"], "trace step 1")
+    close(np.fromfile(out / "2.f32", dtype="<f4").reshape(1, vocab), ref[[35]], TOL["bfloat16"], "trace step 2")
+    cli = subprocess.run([sys.executable, "-m", "kipp_amd.cli", "--model", folder, "--tokens", ",".join(map(str, toks[:9])), "--decode", "5"],
+                         capture_output=True, text=True, timeout=600, cwd=ROOT)
+    assert cli.returncode == 0, cli.stderr[-2000:]
