@@ -319,6 +319,37 @@ def bebulorn_config(qwen: dict, layers: int, kind: str) -> dict:
             "loop": loop, "layers": made}
 
 
+def zivazen_config(qwen: dict, layers: int, kind: str) -> dict:
+    """A Zivazen configuration with the layer sizes of a Qwen3 shape (width, feed-forward, vocabulary) and `layers` layers of
+    one kind, so that every mechanism's kernels stand beside their like alone: "attention" (Qwen3's heads and head size with
+    biases, head norms, a rotation over half the head with stretched frequencies, chunks of 1,024 positions, the added one in
+    the softmax, values mixed with the first layer's; dense feed-forward with biases), "attention_narrow" (the same with
+    values half as wide as the keys), "parallel" (attention with a window of 1,024 keys beside a state space layer of
+    width / 64 heads of 64 with a state of 128 and a filter of 4 taps; dense), "moe" (the attention mixer with a routed
+    feed-forward: 32 experts in 8 groups of which 4 stay, 4 a token, a quarter of the dense inner size each, and a shared
+    one as large), or "mixed" (parallel + dense, attention + routed, parallel + routed, attention + dense)."""
+    width, heads = qwen["hidden_size"], qwen["num_attention_heads"]
+    head_dim = qwen.get("head_dim") or width // heads
+    ff = qwen["intermediate_size"]
+    scaling = {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}
+    attention = {"heads": heads, "kv_heads": qwen["num_key_value_heads"], "dim": head_dim, "vdim": head_dim, "scale": head_dim ** -0.5,
+                 "mask": {"size": 1024}, "rot": {"base": 500000.0, "dims": head_dim // 2, "scaling": scaling}, "v_mix": True}
+    left = {"heads": heads, "kv_heads": qwen["num_key_value_heads"], "dim": head_dim, "vdim": head_dim, "scale": head_dim ** -0.5,
+            "mask": {"size": 1024}, "rot": {"base": 10000.0, "dims": head_dim // 2}}
+    right = {"heads": width // 64, "vdim": 64, "state": 128, "groups": 1, "conv": 4, "norm_groups": 1}
+    parallel = {"left": left, "right": right, "left_scale": 1.2, "right_scale": 1.1}
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "router": {"experts": 32, "top": 4, "groups": {"count": 8, "keep": 4}, "scale": 2.5}, "expert": {"ff": ff // 4},
+           "shared": {"ff": ff // 4}}
+    kinds = {"attention": [("attention", attention, dense)], "attention_narrow": [("attention", dict(attention, vdim=head_dim // 2), dense)],
+             "parallel": [("parallel", parallel, dense)], "moe": [("attention", attention, moe)],
+             "mixed": [("parallel", parallel, dense), ("attention", attention, moe), ("parallel", parallel, moe), ("attention", attention, dense)]}
+    order = kinds[kind]
+    made = [{"type": order[i % len(order)][0], "mixer": json.loads(json.dumps(order[i % len(order)][1])), "mlp": dict(order[i % len(order)][2])}
+            for i in range(layers)]
+    return {"architecture": "Zivazen", "vocab": qwen["vocab_size"], "width": width, "norm": {"eps": 1e-6}, "layers": made}
+
+
 def design_points(config, args, label):
     """Prefill of one 2,048-token prompt and decode steps at two batch sizes behind such prompts, for one model made
     with random weights: milliseconds, tokens a second, and what the kernels ran as (recorded steps, library products,
@@ -406,6 +437,28 @@ def bebulorn_bench(args) -> int:
     return 0
 
 
+def zivazen_bench(args) -> int:
+    """`--design zivazen`: the Zivazen design beside Qwen3 and beside the Bebulorn layers that are closest to its own (windowed
+    attention, the gated delta rule's matrix memory, the routed feed-forward) at equal layer sizes, a few layers of each,
+    random weights: one model for each of its mechanisms alone, and one with all of them in turn."""
+    from kipp_amd.config import shape_config
+    layers = args.layers or 4
+    kinds = args.design_kinds if args.design_kinds != DESIGN_KINDS_DEFAULT else "attention,attention_narrow,parallel,moe,mixed"
+    sizes = {}
+    for shape in [s for s in args.design_shapes.split(",") if s]:
+        qwen = shape_config(shape)
+        qwen["num_hidden_layers"] = layers
+        sizes[shape] = {"qwen3": design_points(qwen, args, f"{shape} qwen3")}
+        for kind in ("attention", "delta", "moe"):
+            sizes[shape][f"bebulorn_{kind}"] = design_points(bebulorn_config(qwen, layers, kind), args, f"{shape} bebulorn, {kind}")
+        for kind in [k for k in kinds.split(",") if k]:
+            sizes[shape][f"zivazen_{kind}"] = design_points(zivazen_config(qwen, layers, kind), args, f"{shape} zivazen, {kind}")
+    print(json.dumps({"metric": "prefill and decode of the Zivazen design beside Qwen3 and Bebulorn's closest layers at equal layer sizes (bf16, random weights)",
+                      "design": "zivazen", "layers": layers, "prompt_tokens": args.prompt, "steps": args.steps,
+                      "unit": "ms and tok/s", "n_gpus": 1, "dtype": "bf16", "data": "synthetic", "sizes": sizes}), flush=True)
+    return 0
+
+
 def design_bench(args) -> int:
     """`--design tobinex`: the Tobinex design beside Qwen3 at equal layer sizes (both with every key kept, and Tobinex
     once more with a window of 1,024 keys behind 4 kept ones), a few layers of each, random weights."""
@@ -445,12 +498,12 @@ def main():
     ap.add_argument("--no-c-host", action="store_true", help="leave out the points measured through the C host")
     ap.add_argument("--products", choices=["default", "own", "auto", "library"], default="default",
                     help="products of many rows (prompt portions): the runtime's default, our kernel only, the fastest of ours and the library's, the library's")
-    ap.add_argument("--design", choices=["tobinex", "rerizen", "bebulorn"], default=None,
+    ap.add_argument("--design", choices=["tobinex", "rerizen", "bebulorn", "zivazen"], default=None,
                     help="instead of the default workload: this design beside Qwen3 at equal layer sizes (prefill and decode, a few layers)")
     ap.add_argument("--design-shapes", default="qwen3-4b,qwen3-8b", help="the Qwen3 shapes whose layer sizes --design takes")
     ap.add_argument("--design-kinds", default=DESIGN_KINDS_DEFAULT,
-                    help="--design rerizen or bebulorn: the models that are measured, one mechanism each or all in turn "
-                         "(bebulorn: attention,lightning,delta,moe,mixed)")
+                    help="--design rerizen, bebulorn or zivazen: the models that are measured, one mechanism each or all in turn "
+                         "(bebulorn: attention,lightning,delta,moe,mixed; zivazen: attention,attention_narrow,parallel,moe,mixed)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -459,6 +512,8 @@ def main():
         return rerizen_bench(args)
     if args.design == "bebulorn":
         return bebulorn_bench(args)
+    if args.design == "zivazen":
+        return zivazen_bench(args)
     if args.design:
         return design_bench(args)
 

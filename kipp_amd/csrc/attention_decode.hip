@@ -128,6 +128,31 @@ __device__ __forceinline__ float2 load_through2(const float* p) {
     return make_float2(__uint_as_float((unsigned)bits), __uint_as_float((unsigned)(bits >> 32)));
 }
 
+// CHUNKED 1: the launcher's `window` is the length of a chunk: the token at position p sees the keys from p - p % window on
+// (chunks are counted from position 0 of the sequence; the splits are planned as for a window of that length).  SINK 1: one
+// more term 2^0 joins the denominator (a key of score 0 that has no value), added once, where a row's result is divided.
+#ifndef CHUNKED
+#define CHUNKED 0
+#endif
+#ifndef SINK
+#define SINK 0
+#endif
+__device__ __forceinline__ int first_key(int pos, int window) {
+#if CHUNKED
+    return pos - pos % window;
+#else
+    return window > 0 ? max(0, pos - window + 1) : 0;
+#endif
+}
+// The added one in the units of a running maximum m (base 2, scale applied): 2^(0 - m).
+__device__ __forceinline__ float sink_term(float m) {
+#if SINK
+    return exp2f(-m);
+#else
+    return 0.0f;
+#endif
+}
+
 // The merge of attention_decode_reduce_kernel (the same sums in the same order) by the workgroup that finished
 // last among the splits of a (token, key/value head): elements `dcol` and `dcol` + 1 (dcol even) of head `head`.
 // A split costs a thread two loads of 8 bytes: its maximum with its denominator, and the two sums.
@@ -166,6 +191,7 @@ __device__ __forceinline__ float2 merge_splits_here(const float* part_acc, const
         a.x += more.x * w;
         a.y += more.y * w;
     }
+    denom += sink_term(m);
     return make_float2(a.x / denom, a.y / denom);
 }
 
@@ -259,7 +285,7 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
     // come last and leave at once instead of holding a place that a working one waits for.
     const int row = rows[blockIdx.x];                 // row of this query token in the batch
     const int pos = positions[row];
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int lo = first_key(pos, window);
     const int first_split = lo / SPLIT_T, last_split = pos / SPLIT_T;
     const int split = first_split + blockIdx.z;
     if (split > last_split) return;                   // the grid covers the longest sequence
@@ -537,7 +563,7 @@ __global__ void __launch_bounds__(THREADS) attention_decode_kernel(
         const int head = kvh * GROUP + g;
         if (n_splits == 1) {
             *(uint32_t*)(out + out_at(row, head * HEAD_DIM + dcol, n_q * HEAD_DIM, FUSED ? pj.out_rows : 0)) =
-                (uint32_t)f32_to_bf16(a0 / s_l[g]) | ((uint32_t)f32_to_bf16(a1 / s_l[g]) << 16);
+                (uint32_t)f32_to_bf16(a0 / (s_l[g] + sink_term(s_m[g]))) | ((uint32_t)f32_to_bf16(a1 / (s_l[g] + sink_term(s_m[g]))) << 16);
         } else {
             put_partial2(arrivals, part_acc, part_ml, ((size_t)blockIdx.x * n_q + head) * max_splits + blockIdx.z, dcol, a0, a1, s_m[g], s_l[g]);
         }
@@ -579,7 +605,7 @@ __global__ void __launch_bounds__(THREADS) attention_decode_stream_kernel(
     const int kvh = blockIdx.y;
     const int row = rows[blockIdx.z];
     const int pos = positions[row];
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int lo = first_key(pos, window);
     const int first_split = lo / BIG, last_split = pos / BIG;
     const int split = first_split + blockIdx.x;
     if (split > last_split) return;
@@ -759,7 +785,7 @@ __global__ void __launch_bounds__(THREADS) attention_decode_stream_kernel(
         for (int w = 0; w < WAVES; ++w) a += s_red[w][g][dcol];
         const int head = kvh * GROUP + g;
         if (n_splits == 1) {
-            out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(a / s_l[g]);
+            out[((size_t)row * n_q + head) * HEAD_DIM + dcol] = f32_to_bf16(a / (s_l[g] + sink_term(s_m[g])));
         } else {
             put_partial(arrivals, part_acc, part_ml, ((size_t)blockIdx.z * n_q + head) * max_splits + blockIdx.x, dcol, a, s_m[g], s_l[g]);
         }
@@ -841,7 +867,7 @@ __global__ void __launch_bounds__(THREADS, 2) attention_decode_ring_kernel(
     const int kvh = blockIdx.y;
     const int row = rows[blockIdx.x];                 // the grid is (query tokens, key/value heads, ranges): ranges beyond a sequence's position come last
     const int pos = positions[row];
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int lo = first_key(pos, window);
     const int first_split = lo / range, last_split = pos / range;
     const int split = first_split + blockIdx.z;
     if (split > last_split) return;
@@ -1078,7 +1104,7 @@ __global__ void __launch_bounds__(THREADS, 2) attention_decode_ring_kernel(
         const int head = kvh * GROUP + g;
         if (n_splits == 1) {
             *(uint32_t*)(out + out_at(row, head * HEAD_DIM + dcol, n_q * HEAD_DIM, FUSED ? pj.out_rows : 0)) =
-                (uint32_t)f32_to_bf16(a0 / l) | ((uint32_t)f32_to_bf16(a1 / l) << 16);
+                (uint32_t)f32_to_bf16(a0 / (l + sink_term(m))) | ((uint32_t)f32_to_bf16(a1 / (l + sink_term(m))) << 16);
         } else {
             put_partial2(arrivals, part_acc, part_ml, ((size_t)blockIdx.x * n_q + head) * max_splits + blockIdx.z, dcol, a0, a1, m, l);
         }
@@ -1098,7 +1124,7 @@ __global__ void attention_decode_reduce_kernel(
     const int head = blockIdx.x, item = blockIdx.y;
     const int row = rows[item];
     const int pos = positions[row];
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int lo = first_key(pos, window);
     const int n_splits = pos / split_keys - lo / split_keys + 1;
     if (n_splits == 1) return;
     const size_t slot0 = ((size_t)item * n_q + head) * max_splits;
@@ -1110,6 +1136,7 @@ __global__ void attention_decode_reduce_kernel(
     m = wave_max(m);
     float denom = 0.0f;
     for (int s = 0; s < n_splits; ++s) denom += part_ml[(slot0 + s) * 2 + 1] * exp2f(part_ml[(slot0 + s) * 2] - m);
+    denom += sink_term(m);
     for (int dcol = threadIdx.x; dcol < HEAD_DIM; dcol += blockDim.x) {
         float a = 0.0f;
         int s = 0;
@@ -1149,7 +1176,7 @@ __global__ void __launch_bounds__(KIPP_WAVE) attention_decode_reduce_few_kernel(
     }
     const int row = rows[item];
     const int pos = positions[row];
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int lo = first_key(pos, window);
     const int n_splits = pos / split_keys - lo / split_keys + 1;
     if (n_splits == 1) return;                                        // written by the attention kernel itself
     // slots of splits that did not run hold whatever was there before: they are chosen away, never multiplied
@@ -1168,6 +1195,7 @@ __global__ void __launch_bounds__(KIPP_WAVE) attention_decode_reduce_few_kernel(
             for (int c = 0; c < COLS; ++c) a[c] += a_s[s][c] * w;
         }
     }
+    denom += sink_term(m);
 #pragma unroll
     for (int c = 0; c < COLS; ++c) {
         const int dcol = lane + KIPP_WAVE * c;
@@ -1335,6 +1363,7 @@ int kipp_attention_decode(const void* q, const void* k_cache, const void* v_cach
     if (head_dim != HEAD_DIM || n_kv <= 0 || n_q != n_kv * GROUP) return -1;
     if (grid_splits <= 0 || grid_splits > max_splits) return -3;
     if (page <= 0 || (page & (page - 1))) return -4;   // pages of a power of two only
+    if (CHUNKED && window <= 0) return -1;
     const float scale_log2e = scale * 1.4426950408889634f;
 #if RING_OK
     {

@@ -45,6 +45,23 @@ __device__ __forceinline__ float capped_score(float s) {
 __device__ __forceinline__ float capped_score(float s) { return s; }
 #endif
 
+// CHUNKED 1: the launcher's `window` is the length of a chunk: a query at position p sees the keys from p - p % window on
+// (chunks are counted from position 0 of the sequence).  SINK 1: one more term 2^0 joins every row's denominator (a key of
+// score 0 that has no value); not with cuts of the keys.
+#ifndef CHUNKED
+#define CHUNKED 0
+#endif
+#ifndef SINK
+#define SINK 0
+#endif
+__device__ __forceinline__ int first_key(int pos, int window) {
+#if CHUNKED
+    return pos - pos % window;
+#else
+    return window > 0 ? max(0, pos - window + 1) : 0;
+#endif
+}
+
 #define BM 128
 #define BN 64
 #define WAVES 4
@@ -119,7 +136,7 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_kernel(
     const bool wave_active = wave * 32 < rows_in_tile;
     const bool row_valid = my_row < rows_in_tile;
     const int my_pos = pos0 + my_row;
-    const int my_lo = window > 0 ? max(0, my_pos - window + 1) : 0;
+    const int my_lo = first_key(my_pos, window);
 
     // the wave's queries as B operand: lane (query l32, half hh) holds q[16 t + 8 hh .. + 7]
     Frag qf[QSTEPS];
@@ -143,7 +160,7 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_kernel(
 
     // with `split_keys` the keys are cut at multiples of it and this work item takes one cut (windows are not split)
     const int split = split_keys > 0 ? item_split[item] : 0;
-    const int tile_lo = split_keys > 0 ? split * (split_keys / BN) : (window > 0 ? max(0, pos0 - window + 1) : 0) / BN;
+    const int tile_lo = split_keys > 0 ? split * (split_keys / BN) : first_key(pos0, window) / BN;
     const int tile_hi = split_keys > 0 ? min(last_pos / BN, (split + 1) * (split_keys / BN) - 1) : last_pos / BN;
 
     // The pages of the keys this workgroup reads, once, into LDS: the loads of a tile then
@@ -312,6 +329,9 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_kernel(
         return;
     }
     // O^T register v of tile dt is column 32 dt + 8 (v / 4) + 4 hh + v % 4 of this lane's query
+#if SINK
+    l_run += __builtin_amdgcn_exp2f(-m_run * scale_log2e);       // the term of score 0, in the units of the running maximum
+#endif
     const float inv = 1.0f / l_run;
     bf16_t* o_row = out + ((size_t)(row0 + my_row) * n_q + head) * HEAD_DIM;
 #pragma unroll
@@ -382,7 +402,7 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_dma_kernel(
     const bool wave_active = wave * 32 < rows_in_tile;
     const bool row_valid = my_row < rows_in_tile;
     const int my_pos = pos0 + my_row;
-    const int my_lo = window > 0 ? max(0, my_pos - window + 1) : 0;
+    const int my_lo = first_key(my_pos, window);
 
     Frag qf[QSTEPS];
 #pragma unroll
@@ -400,7 +420,7 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_dma_kernel(
 
     // with `split_keys` the keys are cut at multiples of it and this work item takes one cut (windows are not split)
     const int split = split_keys > 0 ? item_split[item] : 0;
-    const int tile_lo = split_keys > 0 ? split * (split_keys / BN) : (window > 0 ? max(0, pos0 - window + 1) : 0) / BN;
+    const int tile_lo = split_keys > 0 ? split * (split_keys / BN) : first_key(pos0, window) / BN;
     const int tile_hi = split_keys > 0 ? min(last_pos / BN, (split + 1) * (split_keys / BN) - 1) : last_pos / BN;
     const int page_shift = __builtin_ctz(page);
     const int first_block = (tile_lo * BN) >> page_shift, last_block = min(last_pos, tile_hi * BN + BN - 1) >> page_shift;
@@ -627,6 +647,9 @@ __global__ void __launch_bounds__(THREADS, 2) attention_prefill_dma_kernel(
             }
         return;
     }
+#if SINK
+    l_run += __builtin_amdgcn_exp2f(-m_run * scale_log2e);       // the term of score 0, in the units of the running maximum
+#endif
     const float inv = 1.0f / l_run;
     bf16_t* o_row = out + ((size_t)(row0 + my_row) * n_q + head) * HEAD_DIM;
 #pragma unroll
@@ -709,6 +732,7 @@ int kipp_attention_prefill(const void* q, const void* k_cache, const void* v_cac
     // keys cut at multiples of `split_keys` (0: not cut): work item i then takes cut item_split[i] and writes sums that
     // are not normalised yet into part_acc [rows, n_q, max_splits, head_dim] / part_ml [.., 2]; rows merge_rows[j] with
     // merge_cuts[j] cuts are merged afterwards.  Windows are not cut.
+    if ((CHUNKED && window <= 0) || (SINK && split_keys > 0)) return -1;
     if (split_keys < 0 || (split_keys % BN) || (split_keys > 0 && (window > 0 || !item_split || !part_acc || !part_ml ||
                                                                     max_splits <= 0 || !merge_rows || !merge_cuts)))
         return -8;

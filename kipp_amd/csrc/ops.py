@@ -1105,11 +1105,28 @@ def compute_units(device=None) -> int:
     return COMPUTE_UNITS
 
 
+def attention_build_defines(head_dim: int, group: Optional[int] = None, capped: bool = False, chunked: bool = False, sink: bool = False) -> dict:
+    """The constants of a build of the matrix-core attention kernels (`group` None: the kernel for prompt portions)."""
+    defines = {"HEAD_DIM": head_dim}
+    if group is not None:
+        defines["GROUP"] = group
+    if capped:
+        defines["SOFTCAP"] = 1
+    if chunked:
+        defines["CHUNKED"] = 1
+    if sink:
+        defines["SINK"] = 1
+    return defines
+
+
 def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                      rows: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor,
                      n_q: int, n_kv: int, head_dim: int, scale: float, window: int, max_context: int,
-                     workspace: tuple, grid_splits: Optional[int] = None, capped: bool = False) -> torch.Tensor:
+                     workspace: tuple, grid_splits: Optional[int] = None, capped: bool = False, chunked: bool = False,
+                     sink: bool = False) -> torch.Tensor:
     """Attention of single query tokens (batch rows `rows`) over their pages.
+    `chunked`: the build in which `window` is the length of a chunk: position p sees the keys from p - p % window on.
+    `sink`: the build that adds one to the softmax's denominator (a key of score 0 that has no value).
     `capped`: the build whose scores pass tanh: `scale` is then the cap c, and q comes multiplied by (the score's
     scale / c), so that a weight is exp(c tanh(q . k scale / c) - maximum).
     `max_context`: the longest context among them (sizes the grid); `workspace`:
@@ -1130,9 +1147,8 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     _need(part_acc.dtype == torch.float32 and part_ml.dtype == torch.float32
           and part_acc.numel() >= n_items * n_q * max_splits * head_dim and need <= max_splits,
           "attention_decode: workspace too small for this context")
-    defines = {"HEAD_DIM": head_dim, "GROUP": group}
-    if capped:
-        defines["SOFTCAP"] = 1
+    _need(not chunked or window > 0, "attention_decode: a chunk's length must be positive")
+    defines = attention_build_defines(head_dim, group, capped, chunked, sink)
     fn = _fn("attention_decode", "kipp_attention_decode",
              [_c_ptr] * 10 + [_c_int] * 6 + [_c_float, _c_int, _c_int, _c_int, _c_ptr, _c_ptr], defines)
     _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(part_acc), _ptr(part_ml), _ptr(rows),
@@ -1243,9 +1259,12 @@ def attention_decode_workspace(n_items: int, n_q: int, head_dim: int, max_contex
 def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                       item_seq: torch.Tensor, item_tile: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
                       positions: torch.Tensor, block_table: torch.Tensor, n_q: int, n_kv: int, head_dim: int,
-                      scale: float, window: int = 0, tile_rows: int = 128, cuts=None, capped: bool = False) -> torch.Tensor:
+                      scale: float, window: int = 0, tile_rows: int = 128, cuts=None, capped: bool = False, chunked: bool = False,
+                      sink: bool = False) -> torch.Tensor:
     """Attention of prompt portions: work item i is the `item_tile[i]`-th tile
     of `tile_rows` (128, 64 or 32) query rows of sequence `item_seq[i]`.
+    `chunked`: the build in which `window` is the length of a chunk: position p sees the keys from p - p % window on.
+    `sink`: the build that adds one to the softmax's denominator (a key of score 0 that has no value); not with `cuts`.
     `capped`: the build whose scores pass tanh: `scale` is then the cap c, and q comes multiplied by (the score's
     scale / c), so that a weight is exp(c tanh(q . k scale / c) - maximum).
 
@@ -1262,6 +1281,8 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     _attn_common(q, k_cache, v_cache, out, n_q, n_kv, head_dim, "attention_prefill")
     _need(item_seq.numel() == item_tile.numel(), "attention_prefill: one tile index per work item")
     _need(block_table.shape[1] <= PREFILL_MAX_BLOCKS, "attention_prefill: more pages per sequence than the kernel stages")
+    _need(not chunked or window > 0, "attention_prefill: a chunk's length must be positive")
+    _need(not (sink and cuts is not None), "attention_prefill: the added one in the denominator does not go with cuts of the keys")
     split_keys, item_split, merge_rows, merge_cuts, part_acc, part_ml, max_splits = 0, None, None, None, None, None, 0
     if cuts is not None:
         split_keys, item_split, merge_rows, merge_cuts, (part_acc, part_ml) = cuts
@@ -1276,7 +1297,7 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
               "attention_prefill: cuts need no window, a multiple of 64 keys, one cut per work item and a workspace for every row")
     fn = _fn("attention_prefill", "kipp_attention_prefill",
              [_c_ptr] * 10 + [_c_int] * 6 + [_c_float, _c_int, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int,
-                                             _c_ptr], {"HEAD_DIM": head_dim, "SOFTCAP": 1} if capped else {"HEAD_DIM": head_dim})
+                                             _c_ptr], attention_build_defines(head_dim, None, capped, chunked, sink))
     _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(item_seq), _ptr(item_tile), _ptr(q_start),
               _ptr(q_len), _ptr(positions), _ptr(block_table), block_table.shape[1], item_seq.numel(), n_q, n_kv,
               head_dim, k_cache.shape[2], float(scale), int(window), int(tile_rows), _ptr(item_split), int(split_keys),

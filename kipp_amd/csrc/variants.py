@@ -68,6 +68,7 @@ ATTENTION = [(128, 16), (128, 1), (16, 3), (48, 3), (64, 1), (32, 16), (256, 4),
 EARLY_STREAM = [(128, 4), (48, 3), (16, 2)]      # the kernel for long contexts takes over at 1,024 keys
 WHOLE_CONTEXTS = [(128, 4), (128, 16)]           # the whole-context kernel at few sequences
 CAPPED = [(32, 2), (128, 4), (64, 1), (16, 2), (32, 1)]      # scores capped by tanh: (head size, group)
+CHUNKED = [(32, 2, 1), (128, 4, 1), (64, 1, 1), (64, 3, 0), (16, 4, 1)]      # chunks in the window's place: (head size, group, the added one in the denominator)
 MIXED_HEADS = [(6, 3, 32, 16), (4, 4, 32, 32), (8, 2, 64, 48), (12, 4, 32, 64), (2, 1, 96, 16), (32, 8, 32, 16), (4, 2, 32, 16), (32, 8, 128, 128), (16, 4, 32, 16)]   # (heads, key/value heads, key size, value size) of the attention with mixed heads
 
 
@@ -86,6 +87,12 @@ def check_builds() -> List[Spec]:
         out.append(("attention_decode", {"HEAD_DIM": head_dim, "GROUP": group, "SOFTCAP": 1}))
     out.append(("attention_decode", {"HEAD_DIM": 128, "GROUP": 4, "SOFTCAP": 1, "STREAM_FROM": 1024}))
     out.append(("attention_decode", {"HEAD_DIM": 128, "GROUP": 4, "SOFTCAP": 1, "RING_FROM_PAIRS": 1}))
+    for head_dim, group, sink in CHUNKED:
+        more = {"SINK": 1} if sink else {}
+        out.append(("attention_prefill", {"HEAD_DIM": head_dim, "CHUNKED": 1, **more}))
+        out.append(("attention_decode", {"HEAD_DIM": head_dim, "GROUP": group, "CHUNKED": 1, **more}))
+    out.append(("attention_decode", {"HEAD_DIM": 128, "GROUP": 4, "CHUNKED": 1, "SINK": 1, "STREAM_FROM": 1024}))
+    out.append(("attention_decode", {"HEAD_DIM": 128, "GROUP": 4, "CHUNKED": 1, "SINK": 1, "RING_FROM_PAIRS": 1}))
     from .ops import mixed_attention_builds
     for heads, kv_heads, head_dim, v_dim in MIXED_HEADS:
         out += [("attention_mixed_mfma", defines) for defines in mixed_attention_builds(heads, kv_heads, head_dim, v_dim)]

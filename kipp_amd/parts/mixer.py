@@ -79,13 +79,15 @@ class Attention:
         out = [("rope_kv", None) if spec.plain else ("head_prepare", None), ("attention_generic", None)]
         if not spec.plain and getattr(spec.position, "kind", "none") != "none":
             out.append(("rope_kv", None))       # the step's table of angles
-        if dtype != "bfloat16" or spec.head_dim % 16 or spec.value_dim != spec.head_dim or spec.chunk is not None or spec.sink:
+        if dtype != "bfloat16" or spec.head_dim % 16 or spec.value_dim != spec.head_dim or (spec.sink and spec.chunk is None and spec.window is None):
             return out
+        from ..csrc.ops import attention_build_defines
         group = spec.num_heads // spec.num_kv_heads
-        capped = {"SOFTCAP": 1} if spec.softcap is not None else {}      # capped scores: builds of their own
-        out.append(("attention_prefill", {"HEAD_DIM": spec.head_dim, **capped}))
+        # capped scores, chunks and the added one in the denominator: builds of their own
+        extras = (spec.softcap is not None, spec.chunk is not None, spec.sink)
+        out.append(("attention_prefill", attention_build_defines(spec.head_dim, None, *extras)))
         if group <= 16:
-            out.append(("attention_decode", {"HEAD_DIM": spec.head_dim, "GROUP": group, **capped}))
+            out.append(("attention_decode", attention_build_defines(spec.head_dim, group, *extras)))
         return out
 
     def load(self, tensors):
@@ -174,7 +176,7 @@ class Attention:
 
     def _prefill_work(self, batch):
         """The prefill kernel's work list for this mixer's sizes (`prefill_work`)."""
-        return prefill_work(self.rt, batch, self.spec.num_heads, self.spec.head_dim, self.spec.window)
+        return prefill_work(self.rt, batch, self.spec.num_heads, self.spec.head_dim, self.spec.chunk or self.spec.window)
 
     def _workspace(self, batch):
         """The split decode kernel's partial results for this mixer's sizes (`decode_workspace`)."""
@@ -202,7 +204,9 @@ class Attention:
         norm = "none" if s.qk_norm_eps is None else ("weighted" if s.qk_norm_weight else "plain")
         coef, every = s.q_temp if s.q_temp is not None else (0.0, 0)
         # (without projections of its own only q was projected: its columns stand at the row's start all the same)
-        fast = rt.dtype == "bfloat16" and d % 16 == 0 and d == dv and s.chunk is None and not s.sink \
+        # (with the added one the keys of a prompt portion are never cut, which the matrix-core kernel does only without a
+        # window or chunk)
+        fast = rt.dtype == "bfloat16" and d % 16 == 0 and d == dv and not (s.sink and s.chunk is None and s.window is None) \
             and rt.ops.attention_fast_ok(s.num_heads, s.num_kv_heads, cache.page_size, table.shape[1])
         capped = fast and s.softcap is not None
         # mixed values: the source run leaves its values of this step's tokens for the runs that mix them in
@@ -236,19 +240,21 @@ def paged_attention(rt, batch, q, out, k_cache, v_cache, page_size, table, n_q, 
     which takes values of their own width (`v_cache` may be `k_cache` there too: a value is the first dv numbers
     of its key's row).  `softcap` c > 0: a scaled score s becomes c tanh(s / c) (with `fast`, q must come multiplied by scale / c).  `owner`: a mixer whose `_prefill_work(batch)` and `_workspace(batch)` make the work list and the
     decode workspace (else they are made here for these sizes)."""
-    if fast and (chunk or sink):
-        raise ValueError("the matrix-core attention kernels take a window, not chunks or an added one in the denominator")
     if fast:
-        # capped scores: the builds that pass what they are given through tanh; q then comes times (scale / cap), and the cap is the scale
+        # capped scores: the builds that pass what they are given through tanh; q then comes times (scale / cap), and the cap is the scale.
+        # Chunks: the builds that take the window's place for the chunk's length (work lists and splits are those of a window)
         capped = bool(softcap)
+        span = chunk or window or 0
         if batch.n_portions:
-            item_seq, item_tile, cuts = owner._prefill_work(batch) if owner is not None else prefill_work(rt, batch, n_q, d, window)
+            item_seq, item_tile, cuts = owner._prefill_work(batch) if owner is not None else prefill_work(rt, batch, n_q, d, span or None)
             rt.ops.attention_prefill(q, k_cache, v_cache, out, item_seq, item_tile, batch.q_start, batch.q_len, batch.positions,
-                                     table, n_q, n_kv, d, softcap if capped else scale, window or 0, cuts=cuts, capped=capped)
+                                     table, n_q, n_kv, d, softcap if capped else scale, span, cuts=cuts, capped=capped,
+                                     chunked=bool(chunk), sink=sink)
         if batch.n_decode:
             rt.ops.attention_decode(q, k_cache, v_cache, out, batch.decode_rows, batch.positions, batch.seq_of_token, table,
-                                    n_q, n_kv, d, softcap if capped else scale, window or 0, batch.max_decode_ctx,
-                                    owner._workspace(batch) if owner is not None else decode_workspace(rt, batch, n_q, d), capped=capped)
+                                    n_q, n_kv, d, softcap if capped else scale, span, batch.max_decode_ctx,
+                                    owner._workspace(batch) if owner is not None else decode_workspace(rt, batch, n_q, d), capped=capped,
+                                    chunked=bool(chunk), sink=sink)
     elif d == dv and v_cache is not k_cache and d <= 256 and not softcap and not chunk and not sink:
         # the float32 path, and geometries the matrix-core kernels refuse (groups above 16, odd page sizes)
         rt.ops.paged_attention_generic(q, k_cache, v_cache, out, batch.positions, batch.seq_of_token, table, n_q, n_kv, d,

@@ -310,6 +310,84 @@ def test_squared_relu_experts_biased_activation_and_the_weighted_sum(dtype):
     assert np.allclose(got, x - 0.5 * delta[0], rtol=1e-6, atol=1e-6)
 
 
+@pytest.mark.parametrize("n_q, n_kv, d, page, chunk, sink, build", [
+    (4, 2, 32, 16, 40, True, None), (8, 2, 128, 16, 100, True, None), (3, 3, 64, 8, 7, True, None), (8, 2, 128, 16, 1024, True, None),
+    (6, 2, 64, 16, 300, False, None), (8, 2, 128, 16, 1500, True, "STREAM_FROM"), (8, 2, 128, 16, 300, True, "RING_FROM_PAIRS"),
+    (8, 2, 128, 16, 4096, True, "RING_FROM_PAIRS"), (4, 1, 16, 32, 64, True, None)])
+def test_chunks_and_the_added_one_on_the_matrix_cores(n_q, n_kv, d, page, chunk, sink, build):
+    """The builds of the matrix-core attention in which the window's place is taken by a chunk's length and one is added to the
+    denominator, for prompt portions and for single tokens (also the kernels for long contexts and for whole contexts, built
+    so that small inputs reach them), against the sum written out here; sequence lengths just past, at and just before a
+    chunk's edge."""
+    import torch
+    from kipp_amd.csrc import ops
+    rng = np.random.default_rng(n_q + d + chunk + len(build or ""))
+    scale = 1.7 / np.sqrt(d)
+    seq_lens = [1, 70, 300, 257, 129, chunk + 1, 2 * chunk, 2 * chunk + 1][:5 if chunk > 600 else 8] + ([2300, 1025] if build else [])
+    q_lens = [1, 70, 130, 2, 129, 2, min(chunk, 60) + 1, 3][:5 if chunk > 600 else 8] + ([200, 1] if build else [])
+    q_lens = [min(a, b) for a, b in zip(q_lens, seq_lens)]
+    blocks = [-(-n // page) for n in seq_lens]
+    perm = rng.permutation(sum(blocks) + 3)
+    table = np.zeros((len(seq_lens), max(blocks)), dtype=np.int32)
+    at = 0
+    for i, b in enumerate(blocks):
+        table[i, :b] = perm[at:at + b]
+        at += b
+    k = torch.tensor(rng.normal(size=(len(perm), n_kv, page, d)), dtype=torch.bfloat16)
+    v = torch.tensor(rng.normal(size=(len(perm), n_kv, page, d)) + 1.0, dtype=torch.bfloat16)
+
+    def keys_of(cache, seq, lo, n):
+        return np.stack([cache[table[seq, j // page], :, j % page, :].double().numpy() for j in range(lo, n)])      # [n - lo, n_kv, d]
+
+    def expected(qrow, seq, pos):
+        lo = pos - pos % chunk
+        ks, vs = keys_of(k, seq, lo, pos + 1), keys_of(v, seq, lo, pos + 1)
+        out = np.zeros((n_q, d))
+        for h in range(n_q):
+            g = h // (n_q // n_kv)
+            sc = (ks[:, g] @ qrow[h]) * scale
+            top = max(sc.max(), 0.0)
+            w = np.exp(sc - top)
+            out[h] = (w / (w.sum() + (np.exp(-top) if sink else 0.0))) @ vs[:, g]
+        return out
+
+    inner = ops._fn
+    if build:
+        ops._fn = lambda lib, name, argtypes, defines=None: inner(lib, name, argtypes, dict(defines, **{build: 1024 if build == "STREAM_FROM" else 1}) if lib == "attention_decode" else defines)
+    try:
+        positions, seq_of, q_start = [], [], []
+        for i, (n, ql) in enumerate(zip(seq_lens, q_lens)):
+            q_start.append(len(positions))
+            positions += list(range(n - ql, n))
+            seq_of += [i] * ql
+        t = len(positions)
+        q = torch.tensor(rng.normal(size=(t, n_q * d)), dtype=torch.bfloat16)
+        items = [(i, tile) for i, ql in enumerate(q_lens) for tile in range(-(-ql // 128))]
+        out = ops.attention_prefill(q.cuda(), k.cuda(), v.cuda(), torch.zeros(t, n_q * d, dtype=torch.bfloat16, device="cuda:0"),
+                                    i32([i for i, _ in items]), i32([tile for _, tile in items]), i32(q_start), i32(q_lens), i32(positions),
+                                    i32(table), n_q, n_kv, d, scale, chunk, chunked=True, sink=sink).float().cpu().numpy().reshape(t, n_q, d)
+        qd = q.double().numpy().reshape(t, n_q, d)
+        for row in sorted(set(list(range(0, t, 17)) + q_start + [s + ql - 1 for s, ql in zip(q_start, q_lens)])):
+            ref = expected(qd[row], seq_of[row], positions[row])
+            assert np.abs(out[row] - ref).max() < 2e-2 * max(1.0, np.abs(ref).max()), ("portion", row, seq_of[row], positions[row])
+        n_seq = len(seq_lens)
+        rows = list(range(2, n_seq + 2))
+        pos1, seq1 = [0, 0] + [n - 1 for n in seq_lens], [0, 0] + list(range(n_seq))
+        q1 = torch.tensor(rng.normal(size=(n_seq + 2, n_q * d)), dtype=torch.bfloat16)
+        out1 = torch.zeros(n_seq + 2, n_q * d, dtype=torch.bfloat16, device="cuda:0")
+        ws = ops.attention_decode_workspace(n_seq, n_q, d, max(seq_lens), "cuda:0")
+        ops.attention_decode(q1.cuda(), k.cuda(), v.cuda(), out1, i32(rows), i32(pos1), i32(seq1), i32(table), n_q, n_kv, d, scale, chunk,
+                             max(seq_lens), ws, chunked=True, sink=sink)
+        got = out1.float().cpu().numpy().reshape(n_seq + 2, n_q, d)
+        q1d = q1.double().numpy().reshape(n_seq + 2, n_q, d)
+        for r in rows:
+            ref = expected(q1d[r], seq1[r], pos1[r])
+            assert np.abs(got[r] - ref).max() < 2e-2 * max(1.0, np.abs(ref).max()), ("single token", r, pos1[r])
+        assert not got[:2].any()
+    finally:
+        ops._fn = inner
+
+
 # =============================================================================== the engine
 
 @pytest.mark.parametrize("dtype, page", [("float32", 16), ("bfloat16", 16), ("bfloat16", 32), ("float32", 8)])
