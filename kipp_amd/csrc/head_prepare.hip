@@ -16,7 +16,7 @@
 //     mix     `v_first_out` [tokens][n_kv dv] receives the values as they are here; with `v_first_in` (another layer's,
 //             of the same tokens) the value becomes (1 - lambda) v + lambda v_first, lambda = *v_lambda
 //     write   q to q_out [tokens][n_q d]; the key and value of position p to page table[p / page], slot p % page;
-//             caches [page][kv head][slot][d] and [page][kv head][slot][dv]
+//             caches [page][kv head][slot][d] and [page][kv head][slot][v_row], v_row >= dv (the rest of a row is zeros)
 // All arithmetic is float32.
 #include "common.h"
 #include <math.h>
@@ -33,7 +33,7 @@ __global__ void head_prepare_kernel(
     const float* __restrict__ k_norm_w, float eps, float temp_coef, int temp_every,
     int n_q, int n_kv, int d, int dv, int page, int write_kv, const float* __restrict__ q_head_scale, float v_norm_eps,
     const float* __restrict__ angles, int rotary_dim, const float* __restrict__ v_first_in, float* __restrict__ v_first_out,
-    const float* __restrict__ v_lambda) {
+    const float* __restrict__ v_lambda, int v_row) {
     const int wave = threadIdx.x / KIPP_WAVE;
     const int lane = threadIdx.x & (KIPP_WAVE - 1);
     const int t = blockIdx.y;
@@ -131,11 +131,13 @@ __global__ void head_prepare_kernel(
     } else {
         const int seq = seq_of_token[t];
         const int page_id = block_table[(size_t)seq * max_blocks + pos / page];
-        TC* dst = (kind == 1 ? k_cache : v_cache) + (((size_t)page_id * n_kv + head) * page + pos % page) * width;
+        // a value's row in the cache may be wider than the value (v_row >= dv): the rest is written as zeros
+        const int row = kind == 1 ? d : v_row;
+        TC* dst = (kind == 1 ? k_cache : v_cache) + (((size_t)page_id * n_kv + head) * page + pos % page) * row;
 #pragma unroll
         for (int c = 0; c < MAX_D / KIPP_WAVE; ++c) {
             const int e = lane + c * KIPP_WAVE;
-            if (e < width) store_f(dst, e, vals[c]);
+            if (e < row) store_f(dst, e, e < width ? vals[c] : 0.0f);
         }
     }
 }
@@ -145,9 +147,10 @@ extern "C" int kipp_head_prepare_rotated(
     int cache_dtype, const int32_t* positions, const int32_t* seq_of_token, const int32_t* block_table, int max_blocks,
     int norm_mode, const float* q_norm_w, const float* k_norm_w, float eps, float temp_coef, int temp_every,
     int n_tokens, int n_q, int n_kv, int d, int dv, int page, int write_kv, const float* q_head_scale, float v_norm_eps,
-    const float* angles, int rotary_dim, const float* v_first_in, float* v_first_out, const float* v_lambda,
+    const float* angles, int rotary_dim, const float* v_first_in, float* v_first_out, const float* v_lambda, int v_row,
     hipStream_t stream) {
     if (n_tokens <= 0) return 0;
+    if (v_row < dv || v_row > MAX_D) return -1;
     if (angles != nullptr && (rotary_dim <= 0 || rotary_dim % 2 || rotary_dim > d)) return -1;
     if (v_first_in != nullptr && (v_lambda == nullptr || v_first_in == v_first_out)) return -1;
     if (d <= 0 || d > MAX_D || dv <= 0 || dv > MAX_D || n_q <= 0 || n_kv <= 0 || page <= 0) return -1;
@@ -160,7 +163,7 @@ extern "C" int kipp_head_prepare_rotated(
     hipLaunchKernelGGL((head_prepare_kernel<TO, TC>), grid, block, 0, stream, proj, parts, part_stride, stride, bias, \
                        (TO*)q_out, (TC*)k_cache, (TC*)v_cache, positions, seq_of_token, block_table, max_blocks,      \
                        norm_mode, q_norm_w, k_norm_w, eps, temp_coef, temp_every, n_q, n_kv, d, dv, page, write_kv,     \
-                       q_head_scale, v_norm_eps, angles, rotary_dim, v_first_in, v_first_out, v_lambda)
+                       q_head_scale, v_norm_eps, angles, rotary_dim, v_first_in, v_first_out, v_lambda, v_row)
     if (q_dtype == KIPP_F32 && cache_dtype == KIPP_F32) KIPP_HP(float, float);
     else if (q_dtype == KIPP_BF16 && cache_dtype == KIPP_BF16) KIPP_HP(bf16_t, bf16_t);
     else return -2;
@@ -176,7 +179,7 @@ extern "C" int kipp_head_prepare_scaled(
     hipStream_t stream) {
     return kipp_head_prepare_rotated(proj, parts, stride, bias, q_out, q_dtype, k_cache, v_cache, cache_dtype, positions, seq_of_token,
                                      block_table, max_blocks, norm_mode, q_norm_w, k_norm_w, eps, temp_coef, temp_every, n_tokens, n_q,
-                                     n_kv, d, dv, page, write_kv, q_head_scale, v_norm_eps, nullptr, 0, nullptr, nullptr, nullptr, stream);
+                                     n_kv, d, dv, page, write_kv, q_head_scale, v_norm_eps, nullptr, 0, nullptr, nullptr, nullptr, dv, stream);
 }
 
 extern "C" int kipp_head_prepare(

@@ -451,18 +451,18 @@ def head_prepare(proj: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor,
         _need(q_norm_w is not None and k_norm_w is not None and q_norm_w.dtype == k_norm_w.dtype == torch.float32
               and q_norm_w.numel() == d and k_norm_w.numel() == d, "head_prepare: float32 norm weights [d]")
     _need(k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.shape[:3] == v_cache.shape[:3] and k_cache.shape[1] == n_kv
-          and k_cache.shape[3] == d and v_cache.shape[3] == dv and k_cache.dtype == v_cache.dtype,
-          "head_prepare: caches must be [pages, n_kv, page, d] and [pages, n_kv, page, dv]")
+          and k_cache.shape[3] == d and dv <= v_cache.shape[3] <= 256 and k_cache.dtype == v_cache.dtype,
+          "head_prepare: caches must be [pages, n_kv, page, d] and [pages, n_kv, page, >= dv] (the rest of a value's row is written as zeros)")
     _need(block_table.dim() == 2 and int(temp_every) >= 0, "head_prepare: block_table is [sequences, blocks]")
     fn = _fn("head_prepare", "kipp_head_prepare_rotated",
              [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
-              _c_int, _c_ptr, _c_ptr, _c_float, _c_float, _c_int] + [_c_int] * 7 + [_c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr])
+              _c_int, _c_ptr, _c_ptr, _c_float, _c_float, _c_int] + [_c_int] * 7 + [_c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr])
     _check(fn(_ptr(proj), parts, stride, _ptr(bias), _ptr(q_out), _code(q_out), _ptr(k_cache), _ptr(v_cache), _code(k_cache),
               _ptr(positions), _ptr(seq_of_token), _ptr(block_table), block_table.shape[1],
               {"none": 0, "plain": 1, "weighted": 2}[norm], _ptr(q_norm_w), _ptr(k_norm_w), float(eps), float(temp_coef),
               int(temp_every), n, n_q, n_kv, d, dv, k_cache.shape[2], int(write_kv), _ptr(q_head_scale),
               -1.0 if v_norm_eps is None else float(v_norm_eps), _ptr(angles), int(rotary_dim) if angles is not None else 0,
-              _ptr(v_first_in), _ptr(v_first_out), _ptr(v_lambda), _stream()), "head_prepare")
+              _ptr(v_first_in), _ptr(v_first_out), _ptr(v_lambda), v_cache.shape[3], _stream()), "head_prepare")
     return q_out
 
 

@@ -42,6 +42,12 @@ class Attention:
         self.position = build_part("position", spec.position, runtime)
         self.scale = spec.scale if spec.scale is not None else 1.0 / math.sqrt(spec.head_dim)
         self.w_qkv = self.w_o = self.q_norm = self.k_norm = None
+        # Values narrower than their keys under bfloat16: a value's row in the cache is as wide as a key's, the rest zeros,
+        # so that the matrix-core kernels (which take one head size) run; the output projection gets zero columns to match
+        # (a mixer that reads another run's cache finds that run's rows, padded or not)
+        self.pad_values = runtime.dtype == "bfloat16" and spec.value_dim < spec.head_dim and spec.head_dim % 16 == 0 \
+            and spec.num_heads // spec.num_kv_heads <= 16 and not (spec.sink and spec.chunk is None and spec.window is None)
+        self.w_o_padded = None
 
     @staticmethod
     def params(spec):
@@ -79,8 +85,8 @@ class Attention:
         out = [("rope_kv", None) if spec.plain else ("head_prepare", None), ("attention_generic", None)]
         if not spec.plain and getattr(spec.position, "kind", "none") != "none":
             out.append(("rope_kv", None))       # the step's table of angles
-        if dtype != "bfloat16" or spec.head_dim % 16 or spec.value_dim != spec.head_dim or (spec.sink and spec.chunk is None and spec.window is None):
-            return out
+        if dtype != "bfloat16" or spec.head_dim % 16 or spec.value_dim > spec.head_dim or (spec.sink and spec.chunk is None and spec.window is None):
+            return out      # (values narrower than their keys are cached in rows as wide as the keys: the same builds)
         from ..csrc.ops import attention_build_defines
         group = spec.num_heads // spec.num_kv_heads
         # capped scores, chunks and the added one in the denominator: builds of their own
@@ -100,6 +106,11 @@ class Attention:
         # rows concatenated: one product serves q, k and v; no output element changes
         self.w_qkv = self.rt.weight(torch.cat(rows, dim=0).contiguous())
         self.w_o = self.rt.weight(tensors[names[3]])
+        if self.pad_values:
+            w = tensors[names[3]].reshape(s.hidden_size, s.num_heads, s.value_dim)
+            wide = torch.zeros((s.hidden_size, s.num_heads, s.head_dim), dtype=w.dtype, device=w.device)
+            wide[:, :, :s.value_dim] = w
+            self.w_o_padded = self.rt.weight(wide.reshape(s.hidden_size, s.num_heads * s.head_dim).contiguous())
         if s.qk_norm_eps is not None and s.qk_norm_weight:
             self.q_norm = tensors[names[4]]
             self.k_norm = tensors[names[5]]
@@ -126,7 +137,11 @@ class Attention:
                       page_size=spec.page_size, v_head_dim=spec.v_head_dim)
 
     def cache_need(self):
-        return self.need_of(self.spec)
+        need = self.need_of(self.spec)
+        if self.pad_values:
+            need = KVNeed(num_kv_heads=need.num_kv_heads, head_dim=need.head_dim, window=need.window, page_size=need.page_size,
+                          v_head_dim=None, keep_first=need.keep_first)
+        return need
 
     def state_need(self):
         return None
@@ -206,7 +221,8 @@ class Attention:
         # (without projections of its own only q was projected: its columns stand at the row's start all the same)
         # (with the added one the keys of a prompt portion are never cut, which the matrix-core kernel does only without a
         # window or chunk)
-        fast = rt.dtype == "bfloat16" and d % 16 == 0 and d == dv and not (s.sink and s.chunk is None and s.window is None) \
+        wide_rows = self.pad_values and cache.v.shape[3] == d       # the values lie in rows as wide as the keys
+        fast = rt.dtype == "bfloat16" and d % 16 == 0 and (d == dv or wide_rows) and not (s.sink and s.chunk is None and s.window is None) \
             and rt.ops.attention_fast_ok(s.num_heads, s.num_kv_heads, cache.page_size, table.shape[1])
         capped = fast and s.softcap is not None
         # mixed values: the source run leaves its values of this step's tokens for the runs that mix them in
@@ -225,10 +241,11 @@ class Attention:
                                 angles=angles, rotary_dim=rotary_dim, v_first_in=v_in, v_first_out=v_out, v_lambda=self.v_lambda)
         if rt.dtype == "bfloat16" and not fast:
             rt.generic_attention_launches += 1
-        out = rt.empty((n, s.out_dim), rt.act_dtype)
-        paged_attention(rt, batch, q, out, cache.k, cache.v, cache.page_size, table, s.num_heads, s.num_kv_heads, d, dv,
+        padded = fast and wide_rows             # results as wide as the keys, zeros beyond the value's width
+        out = rt.empty((n, s.q_dim if padded else s.out_dim), rt.act_dtype)
+        paged_attention(rt, batch, q, out, cache.k, cache.v, cache.page_size, table, s.num_heads, s.num_kv_heads, d, d if padded else dv,
                         self.scale, s.window, fast, owner=self, softcap=s.softcap or 0.0, chunk=s.chunk or 0, sink=s.sink)
-        delta = rt.linear(out, self.w_o, slabs=True, defer=True)
+        delta = rt.linear(out, self.w_o_padded if padded else self.w_o, slabs=True, defer=True)
         return delta if self.out_bias is None else WeightedDelta.of(rt, delta, 1.0, self.out_bias)
 
 

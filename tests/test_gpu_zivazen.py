@@ -545,6 +545,31 @@ def test_models_drawn_at_random(tmp_path, seed):
             close(got[rid], plain_logits(folder, toks), 2e-8, f"drawn {seed}/{rid}: {json.dumps(cfg)}")
 
 
+def test_narrow_values_ride_on_the_matrix_cores(tmp_path):
+    """Values narrower than their keys: under bfloat16 their rows in the cache are as wide as the keys (zeros behind the
+    value), every attention launch is a matrix-core one, and logits match the plain implementation under portions and
+    single tokens; under float32 the rows keep the values' own width."""
+    att = lambda heads, kv, dim, vdim, size, **more: dict({"heads": heads, "kv_heads": kv, "dim": dim, "vdim": vdim, "scale": 0.2, "mask": {"size": size},
+                                                           "rot": {"base": 300.0, "dims": 16}}, **more)
+    cfg = {"architecture": "Zivazen", "vocab": 120, "width": 64, "norm": {"eps": 1e-6}, "layers": [
+        {"type": "attention", "mixer": att(4, 2, 32, 16, 50, v_mix=True), "mlp": {"kind": "dense", "ff": 64}},
+        {"type": "parallel", "mixer": {"left": att(4, 1, 64, 32, 33), "right": {"heads": 2, "vdim": 16, "state": 16, "groups": 1, "conv": 2, "norm_groups": 1},
+                                       "left_scale": 1.0, "right_scale": 1.0}, "mlp": None},
+        {"type": "attention", "mixer": att(2, 2, 48, 16, 20, v_mix=True), "mlp": {"kind": "dense", "ff": 64}}]}
+    requests = {"a": H.random_tokens(1, 150, 120), "b": H.random_tokens(2, 37, 120)}
+    for dtype in ("bfloat16", "float32"):
+        folder = write_model(tmp_path / f"narrow-{dtype}", cfg, 3, dtype)
+        engine = engine_of(folder, dtype)
+        widths = [engine.cache.view(run, None).v.shape[3] for run in range(3)]
+        assert widths == ([32, 64, 48] if dtype == "bfloat16" else [16, 32, 16])
+        for steps in (H.whole(requests), H.tail_one_by_one(requests, tail=40)):
+            got = H.replay(engine, requests, steps)
+            for rid, toks in requests.items():
+                close(got[rid], plain_logits(folder, toks), TOL[dtype], f"narrow/{dtype}/{rid}")
+        if dtype == "bfloat16":
+            assert engine.rt.generic_attention_launches == 0
+
+
 def test_recorded_steps_of_a_changing_batch(folders):
     """Three requests decode together from recorded steps while window and chunk pass page borders and the state goes on
     in its slot; one ends early and the batch goes on at another size."""
