@@ -45,10 +45,13 @@ def _rotation(rot: dict, head_dim: int, where: str):
                               high=_float(sc, "high", at), original=_float(sc, "original", at), rotary_dim=dims)
 
 
-def _mask_size(m: dict, where: str) -> int:
-    mask = _get(m, "mask", where)
+def _mask_size(m: dict, where: str) -> Optional[int]:
+    """The length of a chunk or window; None (every earlier position is seen) where the mixer names no mask."""
+    mask = m.get("mask")
+    if mask is None:
+        return None
     _only(mask, ("size",), where + "mask.")
-    return _int(mask, "size", where + "mask.")
+    return _int(mask, "size", where + "mask.") if mask.get("size") is not None else None
 
 
 @dataclass(frozen=True)

@@ -131,8 +131,8 @@ def chunk_attention(cfg, w, prefix, m, h, positions, v_first):
         else:
             lam = float(np.asarray(w[prefix + "vmix"], dtype=DTYPE))
             v = (1.0 - lam) * v + lam * v_first
-    size = m["mask"]["size"]
-    o = attention_core(q, k, v, m["scale"], lambda i, j: positions[i] // size == positions[j] // size, sink=True)
+    size = (m.get("mask") or {}).get("size")        # no mask: every earlier position is seen
+    o = attention_core(q, k, v, m["scale"], lambda i, j: size is None or positions[i] // size == positions[j] // size, sink=True)
     return linear(o.reshape(t_len, heads * dv), w[prefix + "o"], w[prefix + "o.b"]), keep
 
 
@@ -145,8 +145,8 @@ def window_attention(w, prefix, m, h, positions):
     rot = m["rot"]
     freq = rotary_frequencies(rot["dims"], rot["base"], rot.get("scaling"))
     q, k = rotate(q, positions, rot["dims"], freq), rotate(k, positions, rot["dims"], freq)
-    size = m["mask"]["size"]
-    o = attention_core(q, k, v, m["scale"], lambda i, j: positions[i] - positions[j] < size, sink=False)
+    size = (m.get("mask") or {}).get("size")
+    o = attention_core(q, k, v, m["scale"], lambda i, j: size is None or positions[i] - positions[j] < size, sink=False)
     return linear(o.reshape(t_len, heads * dv), w[prefix + "o"])
 
 

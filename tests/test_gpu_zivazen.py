@@ -570,6 +570,22 @@ def test_narrow_values_ride_on_the_matrix_cores(tmp_path):
             assert engine.rt.generic_attention_launches == 0
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mixers_without_a_mask_see_every_earlier_position(tmp_path, dtype):
+    """A configuration whose mixers name no mask: the added one without chunks, the left attention without a window."""
+    att = lambda heads, kv, dim, vdim, **more: dict({"heads": heads, "kv_heads": kv, "dim": dim, "vdim": vdim, "scale": 0.2, "rot": {"base": 300.0, "dims": 16}}, **more)
+    cfg = {"architecture": "Zivazen", "vocab": 120, "width": 64, "norm": {"eps": 1e-6}, "layers": [
+        {"type": "attention", "mixer": att(4, 2, 32, 32, mask=None), "mlp": {"kind": "dense", "ff": 64}},
+        {"type": "parallel", "mixer": {"left": att(4, 2, 32, 32), "right": {"heads": 2, "vdim": 16, "state": 16, "groups": 1, "conv": 2, "norm_groups": 1},
+                                       "left_scale": 1.0, "right_scale": 1.0}, "mlp": None}]}
+    folder = write_model(tmp_path / "open", cfg, 4, dtype)
+    requests = {"a": H.random_tokens(1, 150, 120), "b": H.random_tokens(2, 37, 120)}
+    for steps in (H.whole(requests), H.changing_portions(requests), H.tail_one_by_one(requests, tail=40)):
+        got = H.replay(engine_of(folder, dtype), requests, steps)
+        for rid, toks in requests.items():
+            close(got[rid], plain_logits(folder, toks), TOL[dtype], f"open/{dtype}/{rid}")
+
+
 def test_recorded_steps_of_a_changing_batch(folders):
     """Three requests decode together from recorded steps while window and chunk pass page borders and the state goes on
     in its slot; one ends early and the batch goes on at another size."""

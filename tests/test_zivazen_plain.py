@@ -190,7 +190,7 @@ def test_configuration_keys_and_refusals():
     broken(lambda c: c["layers"][1]["mlp"]["router"].update(top=5))                    # more than the kept groups hold
     broken(lambda c: c["layers"][2]["mixer"].update(vdim=16))                          # cannot be mixed with the first layer's values
     broken(lambda c: c["layers"][0]["mixer"]["rot"].update(dims=7))
-    broken(lambda c: c["layers"][0]["mixer"].pop("mask"))
+    broken(lambda c: c["layers"][0]["mixer"]["mask"].update(size=0))
     broken(lambda c: c.update(loop={"start": 0, "stop": 1, "times": 2}))
 
 
