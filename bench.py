@@ -337,9 +337,9 @@ def zivazen_config(qwen: dict, layers: int, kind: str) -> dict:
     left = {"heads": heads, "kv_heads": qwen["num_key_value_heads"], "dim": head_dim, "vdim": head_dim, "scale": head_dim ** -0.5,
             "mask": {"size": 1024}, "rot": {"base": 10000.0, "dims": head_dim // 2}}
     right = {"heads": width // 64, "vdim": 64, "state": 128, "groups": 1, "conv": 4, "norm_groups": 1}
-    parallel = {"left": left, "right": right, "left_scale": 1.2, "right_scale": 1.1}
+    parallel = {"left": left, "right": right, "left_scale": 1.25, "right_scale": 0.8}
     dense = {"kind": "dense", "ff": ff}
-    moe = {"kind": "moe", "router": {"experts": 32, "top": 4, "groups": {"count": 8, "keep": 4}, "scale": 2.5}, "expert": {"ff": ff // 4},
+    moe = {"kind": "moe", "router": {"experts": 32, "top": 4, "groups": {"count": 8, "keep": 4}, "scale": 2.0}, "expert": {"ff": ff // 4},
            "shared": {"ff": ff // 4}}
     kinds = {"attention": [("attention", attention, dense)], "attention_narrow": [("attention", dict(attention, vdim=head_dim // 2), dense)],
              "parallel": [("parallel", parallel, dense)], "moe": [("attention", attention, moe)],

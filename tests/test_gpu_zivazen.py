@@ -135,7 +135,7 @@ def test_prepared_heads_and_chunked_attention_with_a_key_that_stands_out(dtype, 
     ty = torch.float32 if dtype == "float32" else torch.bfloat16
     rng = np.random.default_rng(d + chunk)
     T, scale, eps, lam = 150, 0.3, 1e-5, 0.35
-    freq = P.rotary_frequencies(rot, 5000.0, {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 64})
+    freq = P.rotary_frequencies(rot, 5000.0, {"factor": 3.0, "low": 1.0, "high": 6.0, "original": 64})
     pages = -(-T // page)
     order = rng.permutation(pages + 3)[:pages]
     table = i32(order.reshape(1, pages))
@@ -273,12 +273,12 @@ def test_grouped_router(experts, top, count, keep, tokens):
     pair_token = torch.empty((tokens * top,), dtype=torch.int32, device="cuda:0")
     place = torch.empty((tokens * top,), dtype=torch.int32, device="cuda:0")
     tiles = torch.empty((ops.moe_max_tiles(tokens, experts, top), 3), dtype=torch.int32, device="cuda:0")
-    ops.moe_route(f32(z), experts, top, 1e-20, chosen, weight, pair_token, place, tiles, router="sigmoid", correction=f32(corr), groups=(count, keep), scale=2.5)
+    ops.moe_route(f32(z), experts, top, 1e-20, chosen, weight, pair_token, place, tiles, router="sigmoid", correction=f32(corr), groups=(count, keep), scale=1.75)
     chosen, weight = chosen.cpu().numpy(), weight.cpu().numpy()
     for t in range(tokens):
-        ref_e, ref_w, margin = P.route(z[t, :experts].astype(np.float64), corr.astype(np.float64), top, count, keep, 2.5)
+        ref_e, ref_w, margin = P.route(z[t, :experts].astype(np.float64), corr.astype(np.float64), top, count, keep, 1.75)
         if margin < 1e-5:
-            assert sorted(chosen[t]) == sorted(set(chosen[t])) and np.isclose(weight[t].sum(), 2.5, rtol=1e-4)
+            assert sorted(chosen[t]) == sorted(set(chosen[t])) and np.isclose(weight[t].sum(), 1.75, rtol=1e-4)
             if t != 3:
                 continue
         assert list(chosen[t]) == ref_e, (t, chosen[t], ref_e)
@@ -505,7 +505,7 @@ def random_configuration(rng):
             size = rng.choice([1, 2, 3])
             keep = rng.randint(1, count)
             mlp = {"kind": "moe", "router": {"experts": count * size, "top": rng.randint(1, min(4, keep * size)), "groups": {"count": count, "keep": keep},
-                                             "scale": rng.choice([1.0, 2.5])}, "expert": {"ff": rng.choice([24, 64, 100])}}
+                                             "scale": rng.choice([1.0, 1.75])}, "expert": {"ff": rng.choice([24, 64, 100])}}
             if rng.random() < 0.6:
                 mlp["shared"] = {"ff": rng.choice([32, 72])}
         if kind == "attention":
@@ -526,7 +526,7 @@ def random_configuration(rng):
             p = rng.choice([8, 16, 40])
             right = {"heads": heads, "vdim": p, "state": rng.choice([8, 16, 48, 130]), "groups": sg, "conv": rng.choice([1, 2, 4, 7]),
                      "norm_groups": rng.choice([1, heads])}
-            mixer = {"left": left, "right": right, "left_scale": rng.choice([1.0, 0.6, 1.2]), "right_scale": rng.choice([1.0, 1.1, 0.3])}
+            mixer = {"left": left, "right": right, "left_scale": rng.choice([1.0, 0.6, 1.3]), "right_scale": rng.choice([1.0, 0.9, 0.3])}
         layers.append({"type": kind, "mixer": mixer, "mlp": mlp})
     return {"architecture": "Zivazen", "vocab": rng.choice([300, 512]), "width": rng.choice([96, 128, 192]),
             "norm": {"eps": rng.choice([1e-5, 1e-6])}, "layers": layers}

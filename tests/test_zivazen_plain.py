@@ -18,14 +18,14 @@ def tiny(name="zivazen-tiny-a"):
 
 def test_rotary_frequencies_by_band():
     """A short wavelength is kept, a long one divided by the factor, one in between blended by its place between them."""
-    sc = {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 100.0}
+    sc = {"factor": 5.0, "low": 1.0, "high": 4.0, "original": 100.0}
     f = P.rotary_frequencies(8, 10000.0, None)
     assert np.allclose(f, [1.0, 0.1, 0.01, 0.001])
     g = P.rotary_frequencies(8, 10000.0, sc)
     # wavelengths 6.28, 62.8, 628, 6283 against 25 and 100
-    assert g[0] == f[0] and g[2] == f[2] / 4 and g[3] == f[3] / 4
+    assert g[0] == f[0] and g[2] == f[2] / 5 and g[3] == f[3] / 5
     s = (100.0 / (2 * math.pi / 0.1) - 1.0) / 3.0
-    assert np.isclose(g[1], (1 - s) * 0.1 / 4 + s * 0.1) and f[1] / 4 < g[1] < f[1]
+    assert np.isclose(g[1], (1 - s) * 0.1 / 5 + s * 0.1) and f[1] / 5 < g[1] < f[1]
 
 
 def test_rotation_turns_halves_and_leaves_the_rest():
