@@ -586,6 +586,25 @@ def test_mixers_without_a_mask_see_every_earlier_position(tmp_path, dtype):
             close(got[rid], plain_logits(folder, toks), TOL[dtype], f"open/{dtype}/{rid}")
 
 
+def test_heads_of_128_turned_whole_decode_from_the_input_product(tmp_path):
+    """The left attention with heads of 128 numbers turned over their whole width and no head norm: single tokens take the
+    kernel that starts from the input product (norm weights absent), prompt portions the rotary kernel's form for whole heads."""
+    att = {"heads": 4, "kv_heads": 2, "dim": 128, "vdim": 128, "scale": 0.09, "mask": {"size": 70}, "rot": {"base": 700.0, "dims": 128}}
+    cfg = {"architecture": "Zivazen", "vocab": 120, "width": 128, "norm": {"eps": 1e-6}, "layers": [
+        {"type": "parallel", "mixer": {"left": att, "right": {"heads": 2, "vdim": 32, "state": 16, "groups": 2, "conv": 3, "norm_groups": 2},
+                                       "left_scale": 0.75, "right_scale": 1.5}, "mlp": {"kind": "dense", "ff": 96}},
+        {"type": "parallel", "mixer": {"left": dict(att, mask={"size": 300}), "right": {"heads": 4, "vdim": 32, "state": 32, "groups": 1, "conv": 4, "norm_groups": 1},
+                                       "left_scale": 1.0, "right_scale": 1.0}, "mlp": None}]}
+    folder = write_model(tmp_path / "whole-heads", cfg, 6, "bfloat16")
+    requests = {"a": H.random_tokens(1, 150, 120), "b": H.random_tokens(2, 37, 120), "c": H.random_tokens(3, 90, 120)}
+    for steps in (H.whole(requests), H.tail_one_by_one(requests, tail=40), H.mixed(requests, seed=2)):
+        engine = engine_of(folder, "bfloat16")
+        got = H.replay(engine, requests, steps)
+        for rid, toks in requests.items():
+            close(got[rid], plain_logits(folder, toks), TOL["bfloat16"], f"whole heads/{rid}")
+        assert engine.rt.generic_attention_launches == 0
+
+
 def test_recorded_steps_of_a_changing_batch(folders):
     """Three requests decode together from recorded steps while window and chunk pass page borders and the state goes on
     in its slot; one ends early and the batch goes on at another size."""
